@@ -1,0 +1,111 @@
+/*
+ * lingua_fp8 -- C ABI of the MI355X (gfx950) float8 linear kernels.
+ *
+ * The reference (facebookresearch/lingua) has no native layer: its float8
+ * path is Python issuing ATen ops.  Each entry point below replaces the ATen
+ * call sequence at the cited lines of the reference's lingua/float8.py and is
+ * what a Python binding (ctypes) of that file binds instead.
+ *
+ * Conventions
+ *   - every pointer is a DEVICE pointer owned by the caller; the library
+ *     allocates nothing, keeps no reference and never synchronises;
+ *   - `stream` is a hipStream_t (NULL = the null stream); work is enqueued on
+ *     it and the call returns at once;
+ *   - bf16 / e4m3 data are passed as `void *` (2-byte / 1-byte elements);
+ *     leading dimensions (`ld*`) are in ELEMENTS;
+ *   - return value: 0 on success, a negative L8_E* code otherwise; the text
+ *     of the last failure on the calling thread is l8_last_error();
+ *   - entry points are re-entrant and thread-safe (forward and autograd
+ *     threads may call concurrently).
+ */
+#ifndef LINGUA_FP8_H
+#define LINGUA_FP8_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define L8_OK 0
+#define L8_EINVAL (-1)  /* bad shape, alignment or null pointer */
+#define L8_EARCH (-2)   /* device is not gfx950 */
+#define L8_EHIP (-3)    /* a HIP runtime call failed */
+
+/* scale modes of l8_gemm_nt */
+#define L8_SCALE_SCALAR 0 /* one fp32 value for the whole operand */
+#define L8_SCALE_ROW 1    /* one fp32 value per row of the operand */
+
+int l8_version(void);
+const char *l8_last_error(void);
+
+/* 0 when `device` (HIP ordinal) is a gfx950 part, L8_EARCH otherwise.  There
+ * is no other code path: callers must fail when this fails. */
+int l8_device_check(int device);
+
+/* Row-wise amax -> scale -> cast.
+ * Replaces lingua/float8.py:86-87 (abs/amax per row) + :43-47 (scale()).
+ *   x        bf16 [R,C], row stride ldx
+ *   q        e4m3fn [R,C], row stride ldq           (may be NULL: amax only)
+ *   scale    fp32 [R] = max(f32(amax),1e-12)/448    (may be NULL with q)
+ *   amax     bf16 [R] row amax, NaN propagating     (may be NULL)
+ *   col_amax fp32 [C] (may be NULL): max-merged (atomically, as non-negative
+ *            float bit patterns) with the column amaxes of x, so that a later
+ *            l8_cast_colwise_transposed() needs no pass of its own to find
+ *            them.  The caller zero-fills it before the first merge.
+ * Requires C % 8 == 0, ldx % 8 == 0, ldq % 8 == 0 and 16-byte aligned x / 8-byte aligned q. */
+int l8_cast_rowwise(const void *x, int64_t R, int64_t C, int64_t ldx,
+                    void *q, int64_t ldq, float *scale, void *amax, float *col_amax,
+                    void *stream);
+
+/* Column amax on its own (same merge semantics as col_amax above). */
+int l8_col_amax(const void *x, int64_t R, int64_t C, int64_t ldx, float *col_amax, void *stream);
+
+/* bf16 amax[n] -> bf16 amax_out[1] = max, NaN propagating.
+ * Replaces lingua/float8.py:115 (tensor amax of the weight from the row
+ * amaxes saved by forward). */
+int l8_amax_reduce(const void *amax, int64_t n, void *amax_out, void *stream);
+
+/* Tensor-wise scale -> cast with a device-resident bf16 amax scalar.
+ * Replaces lingua/float8.py:111 (b_t.t().contiguous()) + :116-118
+ * (repeat_interleave of the scalar) + :43-47 (scale()) for the dgrad weight.
+ *   transpose == 0 : q is [R,C] (ldq >= C);  != 0 : q is [C,R] (ldq >= R)
+ *   scale    fp32 [1]
+ * Requires C % 8 == 0, ldx % 8 == 0. */
+int l8_cast_tensorwise(const void *x, int64_t R, int64_t C, int64_t ldx,
+                       const void *amax, int transpose,
+                       void *q, int64_t ldq, float *scale, void *stream);
+
+/* Column-wise (token-dimension) scale -> cast, written transposed:
+ * equals scale(x.t().contiguous(), its row amax) (lingua/float8.py:43-47 applied to
+ * the operand layout an fp8 wgrad needs; the reference computes wgrad in bf16 at :123).
+ *   col_amax fp32 [C] column amaxes of x (from l8_cast_rowwise / l8_col_amax)
+ *   q        e4m3fn [C,R], row stride ldq;  scale fp32 [C]
+ * Requires C % 8 == 0, ldx % 8 == 0. */
+int l8_cast_colwise_transposed(const void *x, int64_t R, int64_t C, int64_t ldx,
+                               const float *col_amax,
+                               void *q, int64_t ldq, float *scale, void *stream);
+
+/* Scaled fp8 product, both operands reduction-contiguous ("NT"):
+ *   C[m,n] = bf16( (sum_k A[m,k]*B[n,k]) * sa[m or 0] * sb[n or 0] + bias[n] )
+ * fp32 accumulation on the fp8 matrix cores.  Replaces torch._scaled_mm and the
+ * post-scaling around it at lingua/float8.py:65-77 (forward, dgrad) and serves
+ * the fp8 wgrad.
+ *   A e4m3fn [M,K] (lda), B e4m3fn [N,K] (ldb), C bf16 [M,N] (ldc)
+ *   sa_mode / sb_mode: L8_SCALE_SCALAR or L8_SCALE_ROW;  bias bf16 [N] or NULL
+ *   algo: 0 = library default; other values select a tile configuration (see l8_gemm_algo_count)
+ * Requires K % 16 == 0, lda % 16 == 0, ldb % 16 == 0, 16-byte aligned A and B
+ * (the same multiple-of-16 rule torch._scaled_mm enforces). */
+int l8_gemm_nt(const void *A, const void *B, int64_t M, int64_t N, int64_t K,
+               int64_t lda, int64_t ldb,
+               const float *sa, int sa_mode, const float *sb, int sb_mode,
+               const void *bias, void *C, int64_t ldc, int algo, void *stream);
+
+int l8_gemm_algo_count(void);
+/* human-readable description of tile configuration `algo` (1-based), or NULL */
+const char *l8_gemm_algo_name(int algo);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* LINGUA_FP8_H */

@@ -1,0 +1,22 @@
+"""MI355X-native float8 linear path with the API of lingua/float8.py."""
+from .float8 import (  # noqa: F401
+    EPS,
+    Fp8Linear,
+    Fp8LinearFn,
+    config,
+    convert_linears_to_fp8,
+    matmul,
+    named_replace,
+    scale,
+)
+
+__all__ = [
+    "EPS",
+    "Fp8Linear",
+    "Fp8LinearFn",
+    "config",
+    "convert_linears_to_fp8",
+    "matmul",
+    "named_replace",
+    "scale",
+]

@@ -1,0 +1,75 @@
+"""ctypes binding of ``liblingua_fp8.so`` (declared in ``include/lingua_fp8.h``).
+
+There is exactly one implementation: if the shared library is missing, or the
+GPU is not a gfx950 part, every op raises.  Nothing here falls back to PyTorch
+ops or to the CPU.
+"""
+import ctypes
+import os
+import threading
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "liblingua_fp8.so")
+
+_i64 = ctypes.c_int64
+_int = ctypes.c_int
+_p = ctypes.c_void_p
+
+# name -> argtypes; every function returns int except where noted
+SIGNATURES = {
+    "l8_version": [],
+    "l8_last_error": [],
+    "l8_device_check": [_int],
+    "l8_cast_rowwise": [_p, _i64, _i64, _i64, _p, _i64, _p, _p, _p, _p],
+    "l8_col_amax": [_p, _i64, _i64, _i64, _p, _p],
+    "l8_amax_reduce": [_p, _i64, _p, _p],
+    "l8_cast_tensorwise": [_p, _i64, _i64, _i64, _p, _int, _p, _i64, _p, _p],
+    "l8_cast_colwise_transposed": [_p, _i64, _i64, _i64, _p, _p, _i64, _p, _p],
+    "l8_gemm_nt": [_p, _p, _i64, _i64, _i64, _i64, _i64, _p, _int, _p, _int, _p, _p, _i64, _int, _p],
+    "l8_gemm_algo_count": [],
+    "l8_gemm_algo_name": [_int],
+}
+_RETURNS_STR = {"l8_last_error", "l8_gemm_algo_name"}
+
+_lib = None
+_lock = threading.Lock()
+_checked_devices = set()
+
+
+def load():
+    """Load the library (once). Raises RuntimeError when it has not been built."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    with _lock:
+        if _lib is None:
+            if not os.path.exists(LIB_PATH):
+                raise RuntimeError(
+                    f"{LIB_PATH} is missing: build it with `python -m lingua_amd.build` "
+                    "(there is no fallback implementation)"
+                )
+            lib = ctypes.CDLL(LIB_PATH)
+            for name, argtypes in SIGNATURES.items():
+                fn = getattr(lib, name)
+                fn.argtypes = argtypes
+                fn.restype = ctypes.c_char_p if name in _RETURNS_STR else _int
+            _lib = lib
+    return _lib
+
+
+def last_error() -> str:
+    msg = load().l8_last_error()
+    return msg.decode() if msg else ""
+
+
+def check(code: int, what: str) -> None:
+    if code != 0:
+        raise RuntimeError(f"{what} failed ({code}): {last_error()}")
+
+
+def require_device(index: int) -> None:
+    """Raise unless HIP device ``index`` is gfx950 (checked once per device)."""
+    if index in _checked_devices:
+        return
+    check(load().l8_device_check(index), "l8_device_check")
+    _checked_devices.add(index)

@@ -1,0 +1,48 @@
+// Host-side plumbing shared by the entry points: thread-local error text,
+// device identification, cached device properties.
+#include <stdarg.h>
+#include <stdio.h>
+#include <string.h>
+
+#include "l8_common.h"
+
+namespace l8 {
+
+static thread_local char g_err[512] = "";
+
+int fail(int code, const char *fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_err, sizeof(g_err), fmt, ap);
+  va_end(ap);
+  return code;
+}
+
+constexpr int kMaxDev = 64;
+static int g_cus[kMaxDev];  // 0 = not queried yet; benign race: every thread writes the same value
+
+int num_cus() {
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDev) return 256;
+  int c = g_cus[dev];
+  if (c == 0) {
+    if (hipDeviceGetAttribute(&c, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || c <= 0) c = 256;
+    g_cus[dev] = c;
+  }
+  return c;
+}
+
+}  // namespace l8
+
+extern "C" int l8_version(void) { return 1; }
+
+extern "C" const char *l8_last_error(void) { return l8::g_err; }
+
+extern "C" int l8_device_check(int device) {
+  hipDeviceProp_t prop;
+  hipError_t e = hipGetDeviceProperties(&prop, device);
+  if (e != hipSuccess) return l8::fail(L8_EHIP, "hipGetDeviceProperties(%d): %s", device, hipGetErrorString(e));
+  if (strncmp(prop.gcnArchName, "gfx950", 6) != 0)
+    return l8::fail(L8_EARCH, "device %d is %s; this library contains gfx950 code only", device, prop.gcnArchName);
+  return L8_OK;
+}

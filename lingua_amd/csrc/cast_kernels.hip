@@ -1,0 +1,491 @@
+// Fused amax -> fp32 scale -> e4m3fn cast kernels for gfx950 (HBM-bound).
+//
+// Replaces the eager ATen chain of lingua/float8.py:43-47 (scale()), the row
+// amax reductions at :86-87 / :112-114, the tensor amax at :115-118 and the
+// weight transpose copy at :111.  Compulsory traffic per element is 2 bytes
+// read + 1 byte written; every kernel here reads each input byte from HBM once.
+#include "l8_common.h"
+
+namespace l8 {
+
+// ---------------------------------------------------------------------------
+// Row-wise: one wavefront owns one row at a time and keeps it in registers
+// between the amax reduction and the cast.  Lane l of chunk j holds columns
+// [j*512 + l*8, +8) (one 16-byte load, 1 KiB per wave instruction).
+// A workgroup is 4 waves; waves stride over rows so that the optional
+// column-amax by-product is accumulated in registers over many rows and merged
+// once per workgroup (LDS max, then one global atomic max per column).
+// ---------------------------------------------------------------------------
+constexpr int kRowBlock = 256;
+constexpr int kRowWaves = kRowBlock / 64;
+
+template <int NCH>
+L8_DEV void load_row(v4i (&buf)[NCH], const uint16_t *row, int C, int lane) {
+#pragma unroll
+  for (int j = 0; j < NCH; ++j) {
+    const int c = j * 512 + lane * 8;
+    if (c < C) buf[j] = __builtin_nontemporal_load((const v4i *)(row + c));
+    else buf[j] = v4i{0, 0, 0, 0};
+  }
+}
+
+template <int NCH, bool COLMAX>
+__global__ __launch_bounds__(kRowBlock) void cast_rowwise_kernel(
+    const uint16_t *__restrict__ x, int64_t R, int C, int64_t ldx, uint8_t *__restrict__ q, int64_t ldq,
+    float *__restrict__ scale, uint16_t *__restrict__ amax_out, uint32_t *__restrict__ col_amax) {
+  extern __shared__ uint32_t lds_colmax[];  // [C] when COLMAX
+  const int lane = threadIdx.x & 63;
+  const int wave = threadIdx.x >> 6;
+  const int64_t wave_stride = (int64_t)gridDim.x * kRowWaves;
+  int64_t r = (int64_t)blockIdx.x * kRowWaves + wave;
+
+  uint32_t cmax[COLMAX ? NCH * 4 : 1];
+  if (COLMAX) {
+#pragma unroll
+    for (int i = 0; i < NCH * 4; ++i) cmax[i] = 0;
+    for (int c = threadIdx.x; c < C; c += kRowBlock) lds_colmax[c] = 0;
+  }
+
+  v4i cur[NCH];
+  if (r < R) load_row<NCH>(cur, x + r * ldx, C, lane);
+  while (r < R) {
+    const int64_t rn = r + wave_stride;
+    v4i nxt[NCH];
+    if (rn < R) load_row<NCH>(nxt, x + rn * ldx, C, lane);
+
+    // row amax on packed pairs
+    uint32_t m = 0;
+#pragma unroll
+    for (int j = 0; j < NCH; ++j)
+#pragma unroll
+      for (int k = 0; k < 4; ++k) {
+        m = pk_absmax_u16(m, (uint32_t)cur[j][k]);
+        if (COLMAX) cmax[j * 4 + k] = pk_absmax_u16(cmax[j * 4 + k], (uint32_t)cur[j][k]);
+      }
+    m = max(m & 0xffffu, m >> 16);
+    const uint32_t amax_bits = wave_max_u32(m);  // bf16 bits, uniform
+    const bool finite = amax_bits < 0x7f80u;
+    float s;
+    if (finite) {
+      s = scale_from_amax(bf16_bits_to_f32(amax_bits));
+    } else if (amax_bits == 0x7f80u) {
+      s = __uint_as_float(0x7f800000u);  // inf / 448
+    } else {
+      s = __uint_as_float(0x7fc00000u);  // NaN amax -> NaN scale
+    }
+    const float recip = recip_exact(s);
+    if (lane == 0) {
+      if (scale) scale[r] = s;
+      if (amax_out) amax_out[r] = (uint16_t)amax_bits;
+    }
+    if (q) {
+      uint8_t *qrow = q + r * ldq;
+      if (finite) {
+#pragma unroll
+        for (int j = 0; j < NCH; ++j) {
+          const int c = j * 512 + lane * 8;
+          if (c < C) __builtin_nontemporal_store(cvt8(cur[j], recip), (v2i *)(qrow + c));
+        }
+      } else {
+#pragma unroll
+        for (int j = 0; j < NCH; ++j) {
+          const int c = j * 512 + lane * 8;
+          if (c < C) *(v2i *)(qrow + c) = cvt8_slow(cur[j], recip);
+        }
+      }
+    }
+#pragma unroll
+    for (int j = 0; j < NCH; ++j) cur[j] = nxt[j];
+    r = rn;
+  }
+
+  if (COLMAX) {
+    __syncthreads();  // lds_colmax zero-filled
+#pragma unroll
+    for (int j = 0; j < NCH; ++j) {
+      const int c = j * 512 + lane * 8;
+      if (c < C) {
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+          const uint32_t v = cmax[j * 4 + k];
+          atomicMax(&lds_colmax[c + 2 * k], (v & 0xffffu) << 16);       // bf16 -> fp32 bit pattern
+          atomicMax(&lds_colmax[c + 2 * k + 1], v & 0xffff0000u);
+        }
+      }
+    }
+    __syncthreads();
+    for (int c = threadIdx.x; c < C; c += kRowBlock) {
+      const uint32_t v = lds_colmax[c];
+      if (v) atomicMax(&col_amax[c], v);
+    }
+  }
+}
+
+// Fallback for rows too long to keep in registers: two passes over the row by
+// one workgroup (the second pass hits L2).
+__global__ __launch_bounds__(kRowBlock) void cast_rowwise_long_kernel(
+    const uint16_t *__restrict__ x, int64_t R, int C, int64_t ldx, uint8_t *__restrict__ q, int64_t ldq,
+    float *__restrict__ scale, uint16_t *__restrict__ amax_out, uint32_t *__restrict__ col_amax) {
+  __shared__ uint32_t red[kRowWaves];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  for (int64_t r = blockIdx.x; r < R; r += gridDim.x) {
+    const uint16_t *row = x + r * ldx;
+    uint32_t m = 0;
+    for (int c = threadIdx.x * 8; c < C; c += kRowBlock * 8) {
+      const v4i v = *(const v4i *)(row + c);
+#pragma unroll
+      for (int k = 0; k < 4; ++k) {
+        m = pk_absmax_u16(m, (uint32_t)v[k]);
+        if (col_amax) {
+          const uint32_t a = (uint32_t)v[k] & 0x7fff7fffu;
+          if (a & 0xffffu) atomicMax(&col_amax[c + 2 * k], (a & 0xffffu) << 16);
+          if (a >> 16) atomicMax(&col_amax[c + 2 * k + 1], a & 0xffff0000u);
+        }
+      }
+    }
+    m = wave_max_u32(max(m & 0xffffu, m >> 16));
+    __syncthreads();
+    if (lane == 0) red[wave] = m;
+    __syncthreads();
+    uint32_t amax_bits = 0;
+#pragma unroll
+    for (int w = 0; w < kRowWaves; ++w) amax_bits = max(amax_bits, red[w]);
+    float s;
+    if (amax_bits < 0x7f80u) s = scale_from_amax(bf16_bits_to_f32(amax_bits));
+    else s = __uint_as_float(amax_bits == 0x7f80u ? 0x7f800000u : 0x7fc00000u);
+    const float recip = recip_exact(s);
+    if (threadIdx.x == 0) {
+      if (scale) scale[r] = s;
+      if (amax_out) amax_out[r] = (uint16_t)amax_bits;
+    }
+    if (q) {
+      uint8_t *qrow = q + r * ldq;
+      const bool finite = amax_bits < 0x7f80u;
+      for (int c = threadIdx.x * 8; c < C; c += kRowBlock * 8) {
+        const v4i v = *(const v4i *)(row + c);
+        *(v2i *)(qrow + c) = finite ? cvt8(v, recip) : cvt8_slow(v, recip);
+      }
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------
+// Column amax alone: each lane owns 8 columns and walks down a slab of rows.
+// ---------------------------------------------------------------------------
+__global__ __launch_bounds__(256) void col_amax_kernel(const uint16_t *__restrict__ x, int64_t R, int C,
+                                                       int64_t ldx, int rows_per_block,
+                                                       uint32_t *__restrict__ col_amax) {
+  const int c = (blockIdx.x * 256 + threadIdx.x) * 8;
+  if (c >= C) return;
+  const int64_t r0 = (int64_t)blockIdx.y * rows_per_block;
+  const int64_t r1 = (r0 + rows_per_block < R) ? r0 + rows_per_block : R;
+  uint32_t m[4] = {0, 0, 0, 0};
+  for (int64_t r = r0; r < r1; ++r) {
+    const v4i v = __builtin_nontemporal_load((const v4i *)(x + r * ldx + c));
+#pragma unroll
+    for (int k = 0; k < 4; ++k) m[k] = pk_absmax_u16(m[k], (uint32_t)v[k]);
+  }
+#pragma unroll
+  for (int k = 0; k < 4; ++k) {
+    if (m[k] & 0xffffu) atomicMax(&col_amax[c + 2 * k], (m[k] & 0xffffu) << 16);
+    if (m[k] >> 16) atomicMax(&col_amax[c + 2 * k + 1], m[k] & 0xffff0000u);
+  }
+}
+
+// bf16 amax[n] -> bf16 amax_out[1]; one workgroup.
+__global__ __launch_bounds__(256) void amax_reduce_kernel(const uint16_t *__restrict__ amax, int64_t n,
+                                                          uint16_t *__restrict__ out) {
+  __shared__ uint32_t red[4];
+  uint32_t m = 0;
+  for (int64_t i = threadIdx.x; i < n; i += 256) m = max(m, (uint32_t)(amax[i] & 0x7fffu));
+  m = wave_max_u32(m);
+  if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = m;
+  __syncthreads();
+  if (threadIdx.x == 0) out[0] = (uint16_t)max(max(red[0], red[1]), max(red[2], red[3]));
+}
+
+// ---------------------------------------------------------------------------
+// Tensor-wise, same layout out as in: pure streaming.
+// ---------------------------------------------------------------------------
+L8_DEV float scale_from_amax_bits16(uint32_t amax_bits) {
+  if (amax_bits < 0x7f80u) return scale_from_amax(bf16_bits_to_f32(amax_bits));
+  return __uint_as_float(amax_bits == 0x7f80u ? 0x7f800000u : 0x7fc00000u);
+}
+L8_DEV float scale_from_amax_bits32(uint32_t amax_bits) {  // fp32 bit pattern of a non-negative amax
+  if (amax_bits < 0x7f800000u) return scale_from_amax(__uint_as_float(amax_bits));
+  return __uint_as_float(amax_bits == 0x7f800000u ? 0x7f800000u : 0x7fc00000u);
+}
+
+__global__ __launch_bounds__(256) void cast_tensorwise_kernel(const uint16_t *__restrict__ x, int64_t R, int C,
+                                                              int64_t ldx, const uint16_t *__restrict__ amax,
+                                                              uint8_t *__restrict__ q, int64_t ldq,
+                                                              float *__restrict__ scale) {
+  const uint32_t amax_bits = amax[0] & 0x7fffu;
+  const float s = scale_from_amax_bits16(amax_bits);
+  const float recip = recip_exact(s);
+  const bool finite = amax_bits < 0x7f80u;
+  if (blockIdx.x == 0 && threadIdx.x == 0) scale[0] = s;
+  const int cpr = C / 8;  // 16-byte chunks per row
+  const int64_t total = R * cpr;
+  for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < total; i += (int64_t)gridDim.x * 256) {
+    const int64_t r = i / cpr;
+    const int c = (int)(i - r * cpr) * 8;
+    const v4i v = __builtin_nontemporal_load((const v4i *)(x + r * ldx + c));
+    // the amax is handed in and must bound |x|: then every product is within
+    // the finite e4m3 range and the hardware converter agrees with the ATen cast
+    *(v2i *)(q + r * ldq + c) = finite ? cvt8(v, recip) : cvt8_slow(v, recip);
+  }
+}
+
+// ---------------------------------------------------------------------------
+// Transposed casts (tensor-wise for the dgrad weight, column-wise for wgrad):
+// a [128 rows x 64 cols] tile of x becomes a [64 x 128] tile of q.
+// Thread t loads 8 columns (one 16-byte load) from each of 4 consecutive rows,
+// packs, for each of its 8 columns, the 4 row-consecutive e4m3 bytes into one
+// dword and writes it to the transposed tile in LDS; the tile is then read
+// back as 16-byte row segments and stored with full 128-byte output rows.
+// ---------------------------------------------------------------------------
+constexpr int kTR = 128, kTC = 64, kTStride = kTR + 16;  // LDS row stride in bytes
+
+template <bool PER_COL>
+__global__ __launch_bounds__(256) void cast_transposed_kernel(
+    const uint16_t *__restrict__ x, int64_t R, int C, int64_t ldx, const uint16_t *__restrict__ amax_scalar,
+    const uint32_t *__restrict__ col_amax, uint8_t *__restrict__ q, int64_t ldq, float *__restrict__ scale,
+    int vec_store) {
+  __shared__ __attribute__((aligned(16))) uint8_t tile[kTC * kTStride];
+  __shared__ float recips[kTC];
+  const int t = threadIdx.x;
+  const int64_t r0 = (int64_t)blockIdx.y * kTR;
+  const int c0 = blockIdx.x * kTC;
+
+  bool finite = true;
+  if (PER_COL) {
+    if (t < kTC) {
+      const int c = c0 + t;
+      float rc = 0.0f;
+      if (c < C) {
+        const uint32_t bits = col_amax[c];
+        const float s = scale_from_amax_bits32(bits);
+        rc = recip_exact(s);
+        if (bits >= 0x7f800000u) rc = __uint_as_float(0x7fc00000u);  // flag: slow path for this column
+        if (blockIdx.y == 0) scale[c] = s;
+      }
+      recips[t] = rc;
+    }
+    __syncthreads();
+  }
+  float rcp[8];
+  const int cc = t & 7;    // which 8-column chunk of the tile
+  const int rg = t >> 3;   // which 4-row group of the tile (0..31)
+  if (PER_COL) {
+#pragma unroll
+    for (int j = 0; j < 8; ++j) rcp[j] = recips[cc * 8 + j];
+  } else {
+    const uint32_t amax_bits = amax_scalar[0] & 0x7fffu;
+    const float s = scale_from_amax_bits16(amax_bits);
+    finite = amax_bits < 0x7f80u;
+    const float rc = recip_exact(s);
+#pragma unroll
+    for (int j = 0; j < 8; ++j) rcp[j] = rc;
+    if (blockIdx.x == 0 && blockIdx.y == 0 && t == 0) scale[0] = s;
+  }
+
+  // load 4 rows x 8 cols
+  v4i in[4];
+  const int c = c0 + cc * 8;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int64_t r = r0 + rg * 4 + i;
+    if (r < R && c < C) in[i] = __builtin_nontemporal_load((const v4i *)(x + r * ldx + c));
+    else in[i] = v4i{0, 0, 0, 0};
+  }
+  // convert and transpose inside the thread: column j <- rows 0..3
+#pragma unroll
+  for (int j = 0; j < 8; ++j) {
+    const int w = j >> 1;
+    const bool hi = j & 1;
+    float v[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const uint32_t p = (uint32_t)in[i][w];
+      v[i] = __uint_as_float(hi ? (p & 0xffff0000u) : (p << 16)) * rcp[j];
+    }
+    int packed;
+    const bool fast = PER_COL ? (rcp[j] == rcp[j]) : finite;
+    if (fast) {
+      packed = __builtin_amdgcn_cvt_pk_fp8_f32(v[0], v[1], 0, false);
+      packed = __builtin_amdgcn_cvt_pk_fp8_f32(v[2], v[3], packed, true);
+    } else {
+      // non-finite amax: redo the products with the true reciprocal (0 for inf, NaN for NaN)
+      float rc = rcp[j];
+      if (PER_COL) {
+        const uint32_t bits = col_amax[c + j < C ? c + j : 0];
+        rc = recip_exact(scale_from_amax_bits32(bits));
+      }
+      packed = 0;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const uint32_t p = (uint32_t)in[i][w];
+        const float val = __uint_as_float(hi ? (p & 0xffff0000u) : (p << 16)) * rc;
+        packed |= (int)(e4m3fn_from_f32_slow(val) << (8 * i));
+      }
+    }
+    *(int *)(tile + (cc * 8 + j) * kTStride + rg * 4) = packed;
+  }
+  __syncthreads();
+  // write out: 64 output rows (columns of x) x 128 bytes
+#pragma unroll
+  for (int i = 0; i < 2; ++i) {
+    const int oc = (t >> 3) + i * 32;  // output row within the tile
+    const int seg = t & 7;             // 16-byte segment
+    const int col = c0 + oc;
+    const int64_t r = r0 + seg * 16;
+    if (col < C && r < R) {
+      const v4i v = *(const v4i *)(tile + oc * kTStride + seg * 16);
+      uint8_t *dst = q + (int64_t)col * ldq + r;
+      if (vec_store && r + 16 <= R) {
+        __builtin_nontemporal_store(v, (v4i *)dst);
+      } else {
+        const uint8_t *src = tile + oc * kTStride + seg * 16;
+        for (int b = 0; b < 16 && r + b < R; ++b) dst[b] = src[b];
+      }
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------
+// host entry points
+// ---------------------------------------------------------------------------
+template <int NCH>
+static int launch_rowwise(const void *x, int64_t R, int64_t C, int64_t ldx, void *q, int64_t ldq, float *scale,
+                          void *amax, float *col_amax, hipStream_t st) {
+  const int cus = num_cus();
+  int64_t blocks = (R + kRowWaves - 1) / kRowWaves;
+  // with the column-amax by-product fewer, longer-lived workgroups mean fewer merges
+  const int64_t cap = (int64_t)cus * (col_amax ? 4 : 8);
+  if (blocks > cap) blocks = cap;
+  if (col_amax) {
+    const size_t lds = (size_t)C * sizeof(uint32_t);
+    hipLaunchKernelGGL((cast_rowwise_kernel<NCH, true>), dim3((unsigned)blocks), dim3(kRowBlock), lds, st,
+                       (const uint16_t *)x, R, (int)C, ldx, (uint8_t *)q, ldq, scale, (uint16_t *)amax,
+                       (uint32_t *)col_amax);
+  } else {
+    hipLaunchKernelGGL((cast_rowwise_kernel<NCH, false>), dim3((unsigned)blocks), dim3(kRowBlock), 0, st,
+                       (const uint16_t *)x, R, (int)C, ldx, (uint8_t *)q, ldq, scale, (uint16_t *)amax,
+                       (uint32_t *)nullptr);
+  }
+  L8_HIP(hipGetLastError());
+  return L8_OK;
+}
+
+}  // namespace l8
+
+using namespace l8;
+
+static bool aligned(const void *p, size_t a) { return ((uintptr_t)p % a) == 0; }
+
+extern "C" int l8_cast_rowwise(const void *x, int64_t R, int64_t C, int64_t ldx, void *q, int64_t ldq, float *scale,
+                               void *amax, float *col_amax, void *stream) {
+  L8_REQUIRE(R >= 0 && C >= 0, "l8_cast_rowwise: negative shape R=%lld C=%lld", (long long)R, (long long)C);
+  if (R == 0 || C == 0) return L8_OK;
+  L8_REQUIRE(x != nullptr, "l8_cast_rowwise: x is null");
+  L8_REQUIRE((q == nullptr) || (scale != nullptr), "l8_cast_rowwise: q given without scale");
+  L8_REQUIRE(C % 8 == 0 && ldx % 8 == 0 && ldx >= C, "l8_cast_rowwise: C=%lld and ldx=%lld must be multiples of 8, ldx >= C",
+             (long long)C, (long long)ldx);
+  L8_REQUIRE(aligned(x, 16), "l8_cast_rowwise: x must be 16-byte aligned");
+  if (q) L8_REQUIRE(ldq % 8 == 0 && ldq >= C && aligned(q, 8), "l8_cast_rowwise: q must be 8-byte aligned with ldq %% 8 == 0, ldq >= C");
+  L8_REQUIRE(C < (1LL << 31), "l8_cast_rowwise: C too large");
+  hipStream_t st = (hipStream_t)stream;
+  const int64_t nch = (C + 511) / 512;
+  if (nch <= 4) return launch_rowwise<4>(x, R, C, ldx, q, ldq, scale, amax, col_amax, st);
+  if (nch <= 8) return launch_rowwise<8>(x, R, C, ldx, q, ldq, scale, amax, col_amax, st);
+  if (nch <= 16 && !(col_amax && C > 16000)) return launch_rowwise<16>(x, R, C, ldx, q, ldq, scale, amax, col_amax, st);
+  if (nch <= 24 && !(col_amax && C > 16000)) return launch_rowwise<24>(x, R, C, ldx, q, ldq, scale, amax, col_amax, st);
+  int64_t blocks = R < (int64_t)num_cus() * 8 ? R : (int64_t)num_cus() * 8;
+  hipLaunchKernelGGL(cast_rowwise_long_kernel, dim3((unsigned)blocks), dim3(kRowBlock), 0, st, (const uint16_t *)x, R,
+                     (int)C, ldx, (uint8_t *)q, ldq, scale, (uint16_t *)amax, (uint32_t *)col_amax);
+  L8_HIP(hipGetLastError());
+  return L8_OK;
+}
+
+extern "C" int l8_col_amax(const void *x, int64_t R, int64_t C, int64_t ldx, float *col_amax, void *stream) {
+  L8_REQUIRE(R >= 0 && C >= 0, "l8_col_amax: negative shape");
+  if (R == 0 || C == 0) return L8_OK;
+  L8_REQUIRE(x && col_amax, "l8_col_amax: null pointer");
+  L8_REQUIRE(C % 8 == 0 && ldx % 8 == 0 && ldx >= C && aligned(x, 16), "l8_col_amax: C, ldx multiples of 8 and x 16-byte aligned required");
+  L8_REQUIRE(C < (1LL << 31), "l8_col_amax: C too large");
+  const int gx = (int)((C / 8 + 255) / 256);
+  // enough row slabs to fill the chip, at least 64 rows each
+  int64_t slabs = (int64_t)num_cus() * 8 / gx;
+  if (slabs < 1) slabs = 1;
+  int64_t rows_per = (R + slabs - 1) / slabs;
+  if (rows_per < 64) rows_per = 64;
+  slabs = (R + rows_per - 1) / rows_per;
+  L8_REQUIRE(slabs <= 65535, "l8_col_amax: too many row slabs");
+  hipLaunchKernelGGL(col_amax_kernel, dim3(gx, (unsigned)slabs), dim3(256), 0, (hipStream_t)stream,
+                     (const uint16_t *)x, R, (int)C, ldx, (int)rows_per, (uint32_t *)col_amax);
+  L8_HIP(hipGetLastError());
+  return L8_OK;
+}
+
+extern "C" int l8_amax_reduce(const void *amax, int64_t n, void *amax_out, void *stream) {
+  L8_REQUIRE(n >= 1 && amax && amax_out, "l8_amax_reduce: need n >= 1 and non-null pointers");
+  hipLaunchKernelGGL(amax_reduce_kernel, dim3(1), dim3(256), 0, (hipStream_t)stream, (const uint16_t *)amax, n,
+                     (uint16_t *)amax_out);
+  L8_HIP(hipGetLastError());
+  return L8_OK;
+}
+
+static int launch_transposed(bool per_col, const void *x, int64_t R, int64_t C, int64_t ldx, const void *amax,
+                             const float *col_amax, void *q, int64_t ldq, float *scale, hipStream_t st) {
+  const int64_t gx = (C + kTC - 1) / kTC, gy = (R + kTR - 1) / kTR;
+  L8_REQUIRE(gy <= 65535, "transposed cast: R too large (%lld rows)", (long long)R);
+  const int vec = (ldq % 16 == 0 && aligned(q, 16)) ? 1 : 0;
+  if (per_col)
+    hipLaunchKernelGGL((cast_transposed_kernel<true>), dim3((unsigned)gx, (unsigned)gy), dim3(256), 0, st,
+                       (const uint16_t *)x, R, (int)C, ldx, (const uint16_t *)nullptr, (const uint32_t *)col_amax,
+                       (uint8_t *)q, ldq, scale, vec);
+  else
+    hipLaunchKernelGGL((cast_transposed_kernel<false>), dim3((unsigned)gx, (unsigned)gy), dim3(256), 0, st,
+                       (const uint16_t *)x, R, (int)C, ldx, (const uint16_t *)amax, (const uint32_t *)nullptr,
+                       (uint8_t *)q, ldq, scale, vec);
+  L8_HIP(hipGetLastError());
+  return L8_OK;
+}
+
+extern "C" int l8_cast_tensorwise(const void *x, int64_t R, int64_t C, int64_t ldx, const void *amax, int transpose,
+                                  void *q, int64_t ldq, float *scale, void *stream) {
+  L8_REQUIRE(R >= 0 && C >= 0, "l8_cast_tensorwise: negative shape");
+  L8_REQUIRE(amax && scale, "l8_cast_tensorwise: amax and scale must be non-null");
+  if (R == 0 || C == 0) return L8_OK;
+  L8_REQUIRE(x && q, "l8_cast_tensorwise: null pointer");
+  L8_REQUIRE(C % 8 == 0 && ldx % 8 == 0 && ldx >= C && aligned(x, 16), "l8_cast_tensorwise: C, ldx multiples of 8 and x 16-byte aligned required");
+  L8_REQUIRE(C < (1LL << 31), "l8_cast_tensorwise: C too large");
+  hipStream_t st = (hipStream_t)stream;
+  if (transpose) {
+    L8_REQUIRE(ldq >= R, "l8_cast_tensorwise: transposed output needs ldq >= R");
+    return launch_transposed(false, x, R, C, ldx, amax, nullptr, q, ldq, scale, st);
+  }
+  L8_REQUIRE(ldq >= C && ldq % 8 == 0 && aligned(q, 8), "l8_cast_tensorwise: q must be 8-byte aligned with ldq %% 8 == 0, ldq >= C");
+  const int64_t total = R * (C / 8);
+  int64_t blocks = (total + 255) / 256;
+  const int64_t cap = (int64_t)num_cus() * 16;
+  if (blocks > cap) blocks = cap;
+  hipLaunchKernelGGL(cast_tensorwise_kernel, dim3((unsigned)blocks), dim3(256), 0, st, (const uint16_t *)x, R, (int)C,
+                     ldx, (const uint16_t *)amax, (uint8_t *)q, ldq, scale);
+  L8_HIP(hipGetLastError());
+  return L8_OK;
+}
+
+extern "C" int l8_cast_colwise_transposed(const void *x, int64_t R, int64_t C, int64_t ldx, const float *col_amax,
+                                          void *q, int64_t ldq, float *scale, void *stream) {
+  L8_REQUIRE(R >= 0 && C >= 0, "l8_cast_colwise_transposed: negative shape");
+  if (C == 0) return L8_OK;
+  L8_REQUIRE(col_amax && scale, "l8_cast_colwise_transposed: col_amax and scale must be non-null");
+  L8_REQUIRE(R > 0, "l8_cast_colwise_transposed: R must be positive when C > 0");
+  L8_REQUIRE(x && q, "l8_cast_colwise_transposed: null pointer");
+  L8_REQUIRE(C % 8 == 0 && ldx % 8 == 0 && ldx >= C && aligned(x, 16), "l8_cast_colwise_transposed: C, ldx multiples of 8 and x 16-byte aligned required");
+  L8_REQUIRE(ldq >= R, "l8_cast_colwise_transposed: ldq >= R required");
+  L8_REQUIRE(C < (1LL << 31), "l8_cast_colwise_transposed: C too large");
+  return launch_transposed(true, x, R, C, ldx, nullptr, col_amax, q, ldq, scale, (hipStream_t)stream);
+}

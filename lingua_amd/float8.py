@@ -1,0 +1,195 @@
+"""Drop-in for the float8 linear path of facebookresearch/lingua
+(``lingua/float8.py``) on MI355X: same names, arguments and error behaviour,
+with every device operation done by the gfx950 kernels in ``liblingua_fp8.so``.
+
+Mirrors
+  * ``EPS``                          lingua/float8.py:11
+  * ``scale(t, amax_t)``             lingua/float8.py:43-47
+  * ``matmul(...)``                  lingua/float8.py:50-79
+  * ``Fp8LinearFn``                  lingua/float8.py:82-131
+  * ``Fp8Linear``                    lingua/float8.py:134-138
+  * ``named_replace``                lingua/float8.py:141-147
+  * ``convert_linears_to_fp8``       lingua/float8.py:150-191
+
+Differences, all deliberate:
+  * single GPU: the tensor-parallel helpers (``get_splitk``, ``apply_to_partial``
+    and the DTensor back-ports, lingua/float8.py:14-40,194-315) are not here;
+    the number of scale groups per row is always 1;
+  * forward and dgrad round to bf16 once (``bf16(acc * sa * sb + bias)``); the
+    reference's dgrad rounds the unscaled product to bf16 first
+    (lingua/float8.py:59-77), a work-around for a slow CUTLASS kernel;
+  * wgrad is an fp8 product with both operands quantised along the token
+    dimension (``config.fp8_wgrad = True``).  Setting it to False restores the
+    reference's bf16 ``grad_out.t() @ a`` (lingua/float8.py:123);
+  * the Inductor / CUDA-graph side effects of the converter
+    (lingua/float8.py:162,187-189) have no counterpart: nothing here is traced
+    or compiled at run time;
+  * the reference's autograd work-around ``b_t + grad_out[:1,:,None]*0``
+    (lingua/float8.py:108) is a no-op for finite gradients and is not issued.
+"""
+import re
+from dataclasses import dataclass
+from typing import Callable, Optional
+
+import torch
+
+from . import ops
+
+# avoid division by zero when calculating scale (same value as the reference)
+EPS = 1e-12
+
+
+@dataclass
+class Fp8Config:
+    # fp8 wgrad (token-dimension scaling); False = bf16 wgrad as in the reference
+    fp8_wgrad: bool = True
+    # GEMM tile configuration handed to l8_gemm_nt (0 = library default)
+    gemm_algo: int = 0
+
+
+config = Fp8Config()
+
+
+def scale(t: torch.Tensor, amax_t: Optional[torch.Tensor] = None):
+    """Quantise ``t`` [R,C] bf16: returns ``(t_fp8, scale_t)`` like lingua/float8.py:43-47.
+
+    ``amax_t`` selects the granularity by its shape, as the reference's tile
+    broadcast does (lingua/float8.py:24-30): ``[R,1]`` (or None) is row-wise,
+    ``[1,1]`` tensor-wise.  For the row-wise case the amax is recomputed inside
+    the fused kernel (it is a by-product of the same pass), so the values of a
+    given ``[R,1]`` tensor are not read.
+    """
+    if amax_t is None or (amax_t.dim() == 2 and amax_t.shape[0] == t.shape[0] and amax_t.shape[1] == 1 and t.shape[0] != 1):
+        q, s, _ = ops.cast_rowwise(t)
+        return q, s
+    if amax_t.numel() == 1:
+        return ops.cast_tensorwise(t, amax_t.to(torch.bfloat16), transpose=False)
+    raise RuntimeError(f"scale: unsupported amax shape {tuple(amax_t.shape)} for input {tuple(t.shape)}")
+
+
+def matmul(first, amax_first, second_t, amax_second_t, bias, use_fast_accum: bool = True):
+    """lingua/float8.py:50-79: quantise both operands, multiply, scale, add bias.
+
+    ``use_fast_accum`` is accepted for signature parity; accumulation is always
+    fp32 on the matrix cores and the scales are always applied in the epilogue.
+    """
+    del use_fast_accum
+    q1, s1 = scale(first, amax_first)
+    q2, s2 = scale(second_t, amax_second_t)
+    return ops.gemm_nt(q1, q2, s1, s2, bias, algo=config.gemm_algo)
+
+
+class Fp8LinearFn(torch.autograd.Function):
+    """``out = a @ b_t.T + bias`` with fp8 operands (lingua/float8.py:83-131)."""
+
+    @staticmethod
+    def forward(ctx, a, b_t, bias):
+        if a.dtype != torch.bfloat16 or b_t.dtype != torch.bfloat16:
+            raise RuntimeError(f"Fp8LinearFn: bf16 input and weight required, got {a.dtype} and {b_t.dtype}")
+        need_wgrad_stats = config.fp8_wgrad and b_t.requires_grad
+        # column amaxes of `a` fall out of the row-wise pass; wgrad wants them
+        a_col_amax = torch.zeros(a.shape[1], dtype=torch.float32, device=a.device) if need_wgrad_stats else None
+        qa, sa, _ = ops.cast_rowwise(a, col_amax=a_col_amax)
+        qb, sb, amax_b_t = ops.cast_rowwise(b_t)
+        out = ops.gemm_nt(qa, qb, sa, sb, bias, algo=config.gemm_algo)
+
+        ctx.a_requires_grad = a.requires_grad
+        ctx.b_requires_grad = b_t.requires_grad
+        ctx.bias_requires_grad = bias.requires_grad if bias is not None else False
+        ctx.fp8_wgrad = config.fp8_wgrad
+        ctx.gemm_algo = config.gemm_algo
+        ctx.has_col_amax = a_col_amax is not None
+        if a_col_amax is not None:
+            ctx.save_for_backward(a, b_t, amax_b_t, a_col_amax)
+        else:
+            ctx.save_for_backward(a, b_t, amax_b_t)
+        return out
+
+    @staticmethod
+    def backward(ctx, grad_out):
+        if ctx.has_col_amax:
+            a, b_t, amax_b_t, a_col_amax = ctx.saved_tensors
+        else:
+            a, b_t, amax_b_t = ctx.saved_tensors
+            a_col_amax = None
+        if grad_out.dtype != torch.bfloat16:
+            raise RuntimeError(f"Fp8LinearFn.backward: bf16 grad_out required, got {grad_out.dtype}")
+        fp8_wgrad = ctx.fp8_wgrad and ctx.b_requires_grad
+
+        qg = sg = None
+        g_col_amax = None
+        if ctx.a_requires_grad:
+            # grad_out row-wise, weight tensor-wise from the row amaxes saved in
+            # forward, quantised straight into the [K,N] layout dgrad multiplies with
+            g_col_amax = torch.zeros(grad_out.shape[1], dtype=torch.float32, device=grad_out.device) if fp8_wgrad else None
+            qg, sg, _ = ops.cast_rowwise(grad_out, col_amax=g_col_amax)
+            amax_b = ops.amax_reduce(amax_b_t)
+            qb, sb = ops.cast_tensorwise(b_t, amax_b, transpose=True)
+            grad_a = ops.gemm_nt(qg, qb, sg, sb, None, algo=ctx.gemm_algo)
+        else:
+            grad_a = None
+
+        if ctx.b_requires_grad:
+            if fp8_wgrad:
+                if g_col_amax is None:
+                    g_col_amax = ops.col_amax(grad_out)
+                if a_col_amax is None:
+                    a_col_amax = ops.col_amax(a)
+                qgt, sgt = ops.cast_colwise_transposed(grad_out, g_col_amax)
+                qat, sat = ops.cast_colwise_transposed(a, a_col_amax)
+                grad_b = ops.gemm_nt(qgt, qat, sgt, sat, None, algo=ctx.gemm_algo)
+            else:
+                grad_b = grad_out.t() @ a
+        else:
+            grad_b = None
+
+        if ctx.bias_requires_grad:
+            grad_bias = grad_out.sum(dim=0)
+        else:
+            grad_bias = None
+
+        return grad_a, grad_b, grad_bias
+
+
+class Fp8Linear(torch.nn.Linear):
+    def forward(self, input: torch.Tensor) -> torch.Tensor:
+        out = Fp8LinearFn.apply(input.flatten(end_dim=-2), self.weight, self.bias)
+        out = out.unflatten(0, input.shape[:-1])
+        return out
+
+
+def named_replace(fn: Callable[[torch.nn.Module, str], torch.nn.Module], module: torch.nn.Module, name="") -> torch.nn.Module:
+    """Post-order rewrite of a module tree: children first, then the node
+    itself; ``fn`` sees dotted names (``""`` for the root)."""
+    for child_name, child_module in list(module.named_children()):
+        full_name = f"{name}.{child_name}" if name else child_name
+        setattr(module, child_name, named_replace(fn, child_module, full_name))
+    return fn(module, name)
+
+
+def convert_linears_to_fp8(root_module: torch.nn.Module, recipe: str, filter: str) -> torch.nn.Module:
+    """Swap every exact ``nn.Linear`` whose dotted name matches ``filter`` for an
+    ``Fp8Linear`` that shares the same Parameter objects.  Same contract as
+    lingua/float8.py:150-191: unknown recipe -> RuntimeError; a matching
+    subclass of ``nn.Linear`` (e.g. an already converted layer) -> AssertionError."""
+    if recipe not in ["rowwise"]:
+        raise RuntimeError(f"Unknown float8 recipe {recipe!r}")
+
+    filter_re = re.compile(filter)
+
+    def replace(module: torch.nn.Module, name: str) -> torch.nn.Module:
+        if not isinstance(module, torch.nn.Linear) or not filter_re.search(name):
+            return module
+        assert type(module) == torch.nn.Linear, str(type(module))
+        new_module = Fp8Linear(
+            in_features=module.in_features,
+            out_features=module.out_features,
+            bias=module.bias is not None,
+            dtype=module.weight.dtype,
+            device=module.weight.device,
+        )
+        new_module.weight = module.weight
+        new_module.bias = module.bias
+        return new_module
+
+    return named_replace(replace, root_module)

@@ -1,0 +1,141 @@
+"""Tensor-level wrappers around the C ABI: shape checks, output allocation
+(by PyTorch's caching allocator, on the current stream) and the call itself.
+
+All inputs are CUDA (HIP) tensors on a gfx950 device.  Outputs are returned as
+``torch.float8_e4m3fn`` / ``torch.float32`` / ``torch.bfloat16`` tensors.
+"""
+from typing import Optional, Tuple
+
+import torch
+
+from . import _lib
+
+SCALE_SCALAR = 0
+SCALE_ROW = 1
+
+
+def _prep(t: torch.Tensor, what: str):
+    if not t.is_cuda:
+        raise RuntimeError(f"{what}: expected a GPU tensor, got device {t.device} (there is no CPU path)")
+    _lib.require_device(t.device.index)
+    if t.device.index != torch.cuda.current_device():
+        torch.cuda.set_device(t.device)
+    return torch.cuda.current_stream(t.device).cuda_stream
+
+
+def _rows_2d(t: torch.Tensor, dtype, what: str) -> torch.Tensor:
+    if t.dtype != dtype or t.dim() != 2:
+        raise RuntimeError(f"{what}: expected a 2-D {dtype} tensor, got {t.dtype} {tuple(t.shape)}")
+    if t.numel() and (t.stride(1) != 1 or t.stride(0) < t.shape[1]):
+        t = t.contiguous()
+    return t
+
+
+def _ld(t: torch.Tensor) -> int:
+    return t.stride(0) if t.shape[0] > 1 else max(t.shape[1], 1)
+
+
+def cast_rowwise(x: torch.Tensor, col_amax: Optional[torch.Tensor] = None, want_q: bool = True):
+    """Row-wise amax -> scale -> e4m3fn.  Returns (q [R,C] fp8 | None, scale [R,1] fp32, amax [R,1] bf16).
+
+    ``col_amax`` (fp32 [C], zero-initialised by the caller) is max-merged with the column amaxes of x."""
+    x = _rows_2d(x, torch.bfloat16, "cast_rowwise")
+    st = _prep(x, "cast_rowwise")
+    R, C = x.shape
+    q = torch.empty((R, C), dtype=torch.float8_e4m3fn, device=x.device) if want_q else None
+    scale = torch.empty((R, 1), dtype=torch.float32, device=x.device)
+    amax = torch.empty((R, 1), dtype=torch.bfloat16, device=x.device)
+    if col_amax is not None and (col_amax.dtype != torch.float32 or col_amax.numel() != C or not col_amax.is_contiguous()):
+        raise RuntimeError("cast_rowwise: col_amax must be a contiguous fp32 tensor with C elements")
+    code = _lib.load().l8_cast_rowwise(
+        x.data_ptr(), R, C, _ld(x), q.data_ptr() if want_q else None, C, scale.data_ptr(), amax.data_ptr(),
+        col_amax.data_ptr() if col_amax is not None else None, st)
+    _lib.check(code, "l8_cast_rowwise")
+    return q, scale, amax
+
+
+def col_amax(x: torch.Tensor) -> torch.Tensor:
+    """fp32 [C] column amaxes of bf16 x [R,C]."""
+    x = _rows_2d(x, torch.bfloat16, "col_amax")
+    st = _prep(x, "col_amax")
+    R, C = x.shape
+    out = torch.zeros(C, dtype=torch.float32, device=x.device)
+    _lib.check(_lib.load().l8_col_amax(x.data_ptr(), R, C, _ld(x), out.data_ptr(), st), "l8_col_amax")
+    return out
+
+
+def amax_reduce(amax: torch.Tensor) -> torch.Tensor:
+    """bf16 [n] (any shape) -> bf16 [1,1] max, NaN propagating."""
+    if amax.dtype != torch.bfloat16:
+        raise RuntimeError("amax_reduce: expected bf16")
+    amax = amax.contiguous()
+    st = _prep(amax, "amax_reduce")
+    out = torch.empty((1, 1), dtype=torch.bfloat16, device=amax.device)
+    _lib.check(_lib.load().l8_amax_reduce(amax.data_ptr(), amax.numel(), out.data_ptr(), st), "l8_amax_reduce")
+    return out
+
+
+def cast_tensorwise(x: torch.Tensor, amax: torch.Tensor, transpose: bool = False):
+    """Tensor-wise scale -> e4m3fn with a device-resident bf16 amax scalar.
+    Returns (q [R,C] or [C,R] fp8, scale [1,1] fp32)."""
+    x = _rows_2d(x, torch.bfloat16, "cast_tensorwise")
+    st = _prep(x, "cast_tensorwise")
+    if amax.dtype != torch.bfloat16 or amax.numel() != 1 or amax.device != x.device:
+        raise RuntimeError("cast_tensorwise: amax must be a one-element bf16 tensor on the same device")
+    R, C = x.shape
+    q = torch.empty((C, R) if transpose else (R, C), dtype=torch.float8_e4m3fn, device=x.device)
+    scale = torch.empty((1, 1), dtype=torch.float32, device=x.device)
+    code = _lib.load().l8_cast_tensorwise(x.data_ptr(), R, C, _ld(x), amax.data_ptr(), int(transpose),
+                                          q.data_ptr(), max(q.shape[1], 1), scale.data_ptr(), st)
+    _lib.check(code, "l8_cast_tensorwise")
+    return q, scale
+
+
+def cast_colwise_transposed(x: torch.Tensor, col_amax_f32: torch.Tensor):
+    """scale(x.t().contiguous(), its row amax): returns (q [C,R] fp8, scale [C,1] fp32)."""
+    x = _rows_2d(x, torch.bfloat16, "cast_colwise_transposed")
+    st = _prep(x, "cast_colwise_transposed")
+    R, C = x.shape
+    if col_amax_f32.dtype != torch.float32 or col_amax_f32.numel() != C or not col_amax_f32.is_contiguous():
+        raise RuntimeError("cast_colwise_transposed: col_amax must be a contiguous fp32 tensor with C elements")
+    q = torch.empty((C, R), dtype=torch.float8_e4m3fn, device=x.device)
+    scale = torch.empty((C, 1), dtype=torch.float32, device=x.device)
+    code = _lib.load().l8_cast_colwise_transposed(x.data_ptr(), R, C, _ld(x), col_amax_f32.data_ptr(),
+                                                  q.data_ptr(), max(R, 1), scale.data_ptr(), st)
+    _lib.check(code, "l8_cast_colwise_transposed")
+    return q, scale
+
+
+def gemm_nt(qa: torch.Tensor, qb: torch.Tensor, sa: torch.Tensor, sb: torch.Tensor,
+            bias: Optional[torch.Tensor] = None, algo: int = 0, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """bf16( (qa @ qb^T) * sa * sb^T + bias ).  qa [M,K], qb [N,K] fp8; sa [M,1]|[1,1], sb [N,1]|[1,1] fp32."""
+    qa = _rows_2d(qa, torch.float8_e4m3fn, "gemm_nt(A)")
+    qb = _rows_2d(qb, torch.float8_e4m3fn, "gemm_nt(B)")
+    st = _prep(qa, "gemm_nt")
+    M, K = qa.shape
+    N, K2 = qb.shape
+    if K != K2:
+        raise RuntimeError(f"gemm_nt: reduction dims differ ({K} vs {K2})")
+    if sa.dtype != torch.float32 or sb.dtype != torch.float32 or sa.numel() not in (1, M) or sb.numel() not in (1, N):
+        raise RuntimeError("gemm_nt: scales must be fp32 with 1 or M (resp. N) elements")
+    sa, sb = sa.contiguous(), sb.contiguous()
+    sa_mode = SCALE_ROW if sa.numel() == M else SCALE_SCALAR
+    sb_mode = SCALE_ROW if sb.numel() == N else SCALE_SCALAR
+    if bias is not None:
+        if bias.dtype != torch.bfloat16 or bias.numel() != N:
+            raise RuntimeError("gemm_nt: bias must be bf16 with N elements")
+        bias = bias.contiguous()
+    if out is None:
+        out = torch.empty((M, N), dtype=torch.bfloat16, device=qa.device)
+    elif out.dtype != torch.bfloat16 or out.shape != (M, N) or out.stride(1) != 1:
+        raise RuntimeError("gemm_nt: out must be bf16 [M,N] with unit column stride")
+    code = _lib.load().l8_gemm_nt(qa.data_ptr(), qb.data_ptr(), M, N, K, _ld(qa), _ld(qb), sa.data_ptr(), sa_mode,
+                                  sb.data_ptr(), sb_mode, bias.data_ptr() if bias is not None else None,
+                                  out.data_ptr(), _ld(out) if M > 1 else max(N, 1), algo, st)
+    _lib.check(code, "l8_gemm_nt")
+    return out
+
+
+def gemm_algos() -> Tuple[str, ...]:
+    lib = _lib.load()
+    return tuple(lib.l8_gemm_algo_name(i + 1).decode() for i in range(lib.l8_gemm_algo_count()))

@@ -1,0 +1,104 @@
+"""The row-wise float8 recipe as a chain of PyTorch CPU ops -- TEST INFRASTRUCTURE ONLY.
+
+Second, independent restatement of the reference algorithm (the first is the
+integer C code in ``fp8_recipe_oracle.c``).  Every function issues the same
+ATen ops, in the same order and dtypes, as the cited reference lines, with one
+deliberate difference: ``torch._scaled_mm`` with row-wise scales does not exist
+on CPU, so the product is "dequantise, fp32 matmul, round to bf16", which is
+the definition of the expected output that the benchmark spec gives.
+
+This module is also what the benchmark times as ``cpu_baseline`` (kind "port").
+"""
+import torch
+
+EPS = 1e-12  # lingua/float8.py:11
+E4M3_MAX = torch.finfo(torch.float8_e4m3fn).max  # 448.0
+
+
+def row_amax(t: torch.Tensor) -> torch.Tensor:
+    """lingua/float8.py:86 with splitk == 1: [R,C] -> [R,1], same dtype as t."""
+    return t.abs().unflatten(-1, (1, -1)).amax(dim=-1)
+
+
+def tensor_amax_from_rows(amax_rows: torch.Tensor, n_rows_out: int) -> torch.Tensor:
+    """lingua/float8.py:115-118: [N,1] row amaxes -> [n_rows_out,1], all equal to the tensor amax."""
+    a = amax_rows.t().unflatten(-1, (1, -1)).amax(dim=-1)
+    return a.repeat_interleave(n_rows_out // a.shape[0], dim=0, output_size=n_rows_out)
+
+
+def scale(t: torch.Tensor, amax_t: torch.Tensor):
+    """lingua/float8.py:43-47.  amax_t is [R,1] (row-wise) or [1,1] (tensor-wise)."""
+    scale_t = torch.clamp(amax_t.float(), min=EPS) / E4M3_MAX
+    recip = scale_t.reciprocal()
+    # tile broadcast of lingua/float8.py:24-30 for [R,1] and [1,1] scales
+    t_fp8 = (t * recip).to(torch.float8_e4m3fn)
+    return t_fp8, scale_t
+
+
+def dequant_matmul(q1, s1, q2_t, s2_t, bias=None) -> torch.Tensor:
+    """bf16( (q1*s1) @ (q2_t*s2_t)^T + bias ), fp32 throughout."""
+    res = (q1.float() * s1) @ (q2_t.float() * s2_t).t()
+    if bias is not None:
+        res = res + bias.float()
+    return res.to(torch.bfloat16)
+
+
+def matmul(first, amax_first, second_t, amax_second_t, bias=None) -> torch.Tensor:
+    """lingua/float8.py:50-79 (operand roles: both reduction-contiguous)."""
+    q1, s1 = scale(first, amax_first)
+    q2, s2 = scale(second_t, amax_second_t)
+    return dequant_matmul(q1, s1, q2, s2, bias)
+
+
+def linear_forward(a, b_t, bias=None):
+    """lingua/float8.py:85-88"""
+    return matmul(a, row_amax(a), b_t, row_amax(b_t), bias)
+
+
+def linear_dgrad(grad_out, b_t):
+    """lingua/float8.py:110-119"""
+    amax_b_t = row_amax(b_t)
+    b = b_t.t().contiguous()
+    amax_b = tensor_amax_from_rows(amax_b_t, b.shape[0])
+    return matmul(grad_out, row_amax(grad_out), b, amax_b)
+
+
+def linear_wgrad_bf16(grad_out, a):
+    """lingua/float8.py:123"""
+    return grad_out.t() @ a
+
+
+def linear_wgrad_fp8(grad_out, a):
+    """fp8 wgrad (not in the reference): the recipe's scale() applied to the
+    operands transposed so that the token dimension is the reduction one."""
+    gt = grad_out.t().contiguous()
+    at = a.t().contiguous()
+    return matmul(gt, row_amax(gt), at, row_amax(at))
+
+
+def linear_fwd_bwd(a, b_t, grad_out, bias=None, wgrad_fp8=True):
+    out = linear_forward(a, b_t, bias)
+    grad_a = linear_dgrad(grad_out, b_t)
+    grad_b = linear_wgrad_fp8(grad_out, a) if wgrad_fp8 else linear_wgrad_bf16(grad_out, a)
+    grad_bias = grad_out.sum(dim=0) if bias is not None else None  # lingua/float8.py:127
+    return out, grad_a, grad_b, grad_bias
+
+
+def swiglu_mlp_fwd_bwd(x, w1, w2, w3, grad_y):
+    """SwiGLU MLP of lingua/transformer.py:469-471 with every linear in fp8,
+    forward and backward; elementwise work in bf16 as eager PyTorch does it."""
+    x1 = linear_forward(x, w1)
+    x3 = linear_forward(x, w3)
+    h = torch.nn.functional.silu(x1) * x3
+    y = linear_forward(h, w2)
+    # backward
+    dh = linear_dgrad(grad_y, w2)
+    dw2 = linear_wgrad_fp8(grad_y, h)
+    x1f, x3f, dhf = x1.float(), x3.float(), dh.float()
+    sig = torch.sigmoid(x1f)
+    dx3 = (dhf * (x1f * sig)).to(torch.bfloat16)
+    dx1 = (dhf * x3f * (sig * (1 + x1f * (1 - sig)))).to(torch.bfloat16)
+    dx = (linear_dgrad(dx1, w1).float() + linear_dgrad(dx3, w3).float()).to(torch.bfloat16)
+    dw1 = linear_wgrad_fp8(dx1, x)
+    dw3 = linear_wgrad_fp8(dx3, x)
+    return y, dx, dw1, dw2, dw3

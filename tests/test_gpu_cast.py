@@ -1,0 +1,221 @@
+"""GPU parity of the cast kernels against the CPU oracle: e4m3 bytes, fp32
+scales and bf16 amaxes must be bit-identical (NaN codes compare equal
+irrespective of sign, see golden_util.fp8_equal_mod_nan_sign)."""
+import pytest
+import torch
+
+import oracle
+from conftest import seeded_bf16
+from golden_util import bits_equal, fp8_equal_mod_nan_sign, load_golden
+
+pytestmark = pytest.mark.gpu
+
+
+def dev(t):
+    return t.to("cuda")
+
+
+def check_rowwise(x, with_col=False):
+    from lingua_amd import ops
+    col = torch.zeros(x.shape[1], dtype=torch.float32, device="cuda") if with_col else None
+    q, s, a = ops.cast_rowwise(dev(x), col_amax=col)
+    qo, so, ao = oracle.cast_rowwise(x)
+    assert torch.equal(q.cpu().view(torch.uint8), qo), "bytes differ"
+    assert bits_equal(s.cpu().reshape(-1), so), "scales differ"
+    assert bits_equal(a.cpu().reshape(-1), ao), "amax differ"
+    if with_col:
+        assert bits_equal(col.cpu(), oracle.col_amax(x).float()), "column amax differ"
+    return q, s
+
+
+def test_golden_vectors():
+    from lingua_amd import ops
+    g = load_golden()
+    for name, t in (("x", g["x"]), ("w", g["w"]), ("g", g["go"])):
+        q, s, a = ops.cast_rowwise(dev(t))
+        assert torch.equal(q.cpu().view(torch.uint8), g["q_" + name]), name
+        assert bits_equal(s.cpu().reshape(-1), g["s_" + name]), name
+    assert bits_equal(ops.cast_rowwise(dev(g["x"]))[2].cpu().reshape(-1), g["amax_x"])
+    w = dev(g["w"])
+    _, _, amax_w = ops.cast_rowwise(w, want_q=False)
+    qwt, swt = ops.cast_tensorwise(w, ops.amax_reduce(amax_w), transpose=True)
+    assert torch.equal(qwt.cpu().view(torch.uint8), g["q_wt"])
+    assert bits_equal(swt.cpu().reshape(-1).expand(g["s_wt"].shape).contiguous(), g["s_wt"])
+    for name, t in (("gt", g["go"]), ("xt", g["x"])):
+        td = dev(t)
+        q, s = ops.cast_colwise_transposed(td, ops.col_amax(td))
+        assert torch.equal(q.cpu().view(torch.uint8), g["q_" + name]), name
+        assert bits_equal(s.cpu().reshape(-1), g["s_" + name]), name
+    x = dev(g["x"])
+    q, s = ops.cast_tensorwise(x, ops.amax_reduce(ops.cast_rowwise(x, want_q=False)[2]))
+    assert torch.equal(q.cpu().view(torch.uint8), g["q_x_tw"]) and bits_equal(s.cpu().reshape(-1), g["s_x_tw"])
+
+
+@pytest.mark.parametrize("shape", [(1, 8), (3, 16), (7, 520), (5, 4096), (300, 2048), (33, 11008), (9, 12288),
+                                   (1027, 1024), (3, 16384), (2, 40000)])
+@pytest.mark.parametrize("with_col", [False, True])
+def test_rowwise_shapes(shape, with_col):
+    x = seeded_bf16(shape, seed=shape[0] * 131 + shape[1])
+    x[0, 0] = 0.0
+    if shape[0] > 2:
+        x[2] = 0.0
+    check_rowwise(x, with_col)
+
+
+def test_rowwise_config1_inputs():
+    check_rowwise(seeded_bf16((4096, 2048), 1.0, seed=0), with_col=True)
+    check_rowwise(seeded_bf16((2048, 2048), 0.02, seed=1))
+
+
+def test_rowwise_strided_input_and_col_amax_merge():
+    from lingua_amd import ops
+    big = seeded_bf16((64, 1536), seed=9)
+    x = big[:, 256:256 + 1024]              # row stride 1536, offset 512 bytes
+    xd = dev(big)[:, 256:256 + 1024]
+    col = torch.full((1024,), 0.5, dtype=torch.float32, device="cuda")
+    q, s, a = ops.cast_rowwise(xd, col_amax=col)
+    qo, so, ao = oracle.cast_rowwise(x.contiguous())
+    assert torch.equal(q.cpu().view(torch.uint8), qo) and bits_equal(s.cpu().reshape(-1), so)
+    want = torch.maximum(oracle.col_amax(x.contiguous()).float(), torch.tensor(0.5))
+    assert bits_equal(col.cpu(), want)
+
+
+def test_rowwise_nonfinite_rows():
+    from lingua_amd import ops
+    x = seeded_bf16((6, 1024), seed=4)
+    x[1, 3] = float("inf")
+    x[2, 5] = float("nan")
+    x[3, 7] = float("-inf")
+    x[3, 9] = float("nan")
+    q, s, a = ops.cast_rowwise(dev(x))
+    qo, so, ao = oracle.cast_rowwise(x)
+    assert fp8_equal_mod_nan_sign(q, qo)
+    s, a = s.cpu().reshape(-1), a.cpu().reshape(-1)
+    assert torch.equal(s.isnan(), so.isnan()) and torch.equal(s.isinf(), so.isinf())
+    fin = so.isfinite()
+    assert bits_equal(s[fin], so[fin])
+    assert torch.equal(a.isnan(), ao.isnan()) and bits_equal(a[~ao.isnan()], ao[~ao.isnan()])
+
+
+@pytest.mark.parametrize("amax", [448.0, 1.0, 0.0123, 3.3895e38, 1e-30, 240.0, 5.5e-13, 7.0])
+def test_every_bf16_pattern_through_the_hardware_converter(amax):
+    # one row per 4096 patterns; each row's amax is forced to `amax`, larger magnitudes and NaNs are zeroed
+    bits = torch.arange(0, 65536, dtype=torch.int32).to(torch.int16)
+    x = bits.view(torch.bfloat16).clone().reshape(16, 4096)
+    a = torch.tensor(amax).to(torch.bfloat16)
+    bad = ~(x.float().abs() <= a.float())
+    x[bad] = 0.0
+    x[:, 0] = a
+    check_rowwise(x)
+    # same patterns as one long row (two-pass kernel) and through the transposed kernels
+    from lingua_amd import ops
+    long_row = x.reshape(1, -1)
+    check_rowwise(long_row)
+    xd = dev(x)
+    qt, st = ops.cast_colwise_transposed(xd, ops.col_amax(xd))
+    qo, so = oracle.cast_colwise_transposed(x)
+    assert torch.equal(qt.cpu().view(torch.uint8), qo) and bits_equal(st.cpu().reshape(-1), so)
+    qw, sw = ops.cast_tensorwise(xd, dev(a.reshape(1, 1)))
+    qwo, swo = oracle.cast_tensorwise(x, a)
+    assert torch.equal(qw.cpu().view(torch.uint8), qwo) and bits_equal(sw.cpu().reshape(-1), swo)
+
+
+@pytest.mark.parametrize("shape", [(1, 8), (4, 8), (128, 64), (129, 72), (100, 200), (257, 1000), (2048, 512),
+                                   (50, 11008), (1030, 136)])
+def test_transposed_kernels_shapes(shape):
+    from lingua_amd import ops
+    x = seeded_bf16(shape, seed=shape[0] * 7 + shape[1])
+    x[0, 0] = 0.0
+    if shape[1] > 16:
+        x[:, 11] = 0.0  # an all-zero column: scale floor
+    xd = dev(x)
+    ca = ops.col_amax(xd)
+    assert bits_equal(ca.cpu(), oracle.col_amax(x).float())
+    q, s = ops.cast_colwise_transposed(xd, ca)
+    qo, so = oracle.cast_colwise_transposed(x)
+    assert torch.equal(q.cpu().view(torch.uint8), qo) and bits_equal(s.cpu().reshape(-1), so)
+    amax = ops.amax_reduce(ops.cast_rowwise(xd, want_q=False)[2])
+    assert bits_equal(amax.cpu().reshape(()), oracle.amax_of_amaxes(oracle.row_amax(x)))
+    for tr in (False, True):
+        q, s = ops.cast_tensorwise(xd, amax, transpose=tr)
+        qo, so = oracle.cast_tensorwise(x, transpose=tr)
+        assert torch.equal(q.cpu().view(torch.uint8), qo), tr
+        assert bits_equal(s.cpu().reshape(-1), so), tr
+
+
+def test_colwise_nonfinite_columns():
+    from lingua_amd import ops
+    x = seeded_bf16((40, 64), seed=6)
+    x[3, 5] = float("inf")
+    x[7, 9] = float("nan")
+    xd = dev(x)
+    q, s = ops.cast_colwise_transposed(xd, ops.col_amax(xd))
+    qo, so = oracle.cast_colwise_transposed(x)
+    assert fp8_equal_mod_nan_sign(q, qo)
+    s = s.cpu().reshape(-1)
+    assert s[5].isinf() and s[9].isnan()
+    fin = so.isfinite()
+    assert bits_equal(s[fin], so[fin])
+
+
+def outlier_stress_input(rows=16384, cols=4096, seed=0):
+    """Student-t (df=3) activations, 0.1 % of channels x100, 1 % of rows all-zero."""
+    g = torch.Generator().manual_seed(seed)
+    z = torch.randn(rows, cols, generator=g)
+    chi = torch.randn(3, rows, cols, generator=g).pow_(2).sum(0)
+    x = z / (chi / 3.0).sqrt_()
+    del z, chi
+    ch = torch.randperm(cols, generator=g)[: max(1, cols // 1000)]
+    x[:, ch] *= 100.0
+    zr = torch.randperm(rows, generator=g)[: max(1, rows // 100)]
+    x[zr] = 0.0
+    return x.to(torch.bfloat16), ch, zr
+
+
+def test_outlier_stress_full_size_rowwise_tensorwise_colwise():
+    from lingua_amd import ops
+    x, ch, zr = outlier_stress_input()
+    xd = dev(x)
+    col = torch.zeros(x.shape[1], dtype=torch.float32, device="cuda")
+    q, s, a = ops.cast_rowwise(xd, col_amax=col)
+    qo, so, ao = oracle.cast_rowwise(x)
+    assert torch.equal(q.cpu().view(torch.uint8), qo)
+    assert bits_equal(s.cpu().reshape(-1), so) and bits_equal(a.cpu().reshape(-1), ao)
+    assert (s.cpu().reshape(-1)[zr].view(torch.int32) == 0x2720D7C5).all()
+    assert (q.cpu().view(torch.uint8)[zr] == 0).all()
+    assert bits_equal(col.cpu(), oracle.col_amax(x).float())
+    amax = ops.amax_reduce(a)
+    qt, st = ops.cast_tensorwise(xd, amax)
+    qto, sto = oracle.cast_tensorwise(x)
+    assert torch.equal(qt.cpu().view(torch.uint8), qto) and bits_equal(st.cpu().reshape(-1), sto)
+    qc, sc = ops.cast_colwise_transposed(xd, col)
+    qco, sco = oracle.cast_colwise_transposed(x)
+    assert torch.equal(qc.cpu().view(torch.uint8), qco) and bits_equal(sc.cpu().reshape(-1), sco)
+    # row-wise scaling keeps far more of the signal than one scale for the whole tensor
+    xf = x.float()
+    deq_r = q.cpu().float() * s.cpu()
+    deq_t = qt.cpu().float() * st.cpu()
+    err_r = (deq_r - xf).norm() / xf.norm()
+    err_t = (deq_t - xf).norm() / xf.norm()
+    assert err_r < err_t
+
+
+def test_ffn_hidden_shape_properties_full_size():
+    # [16384, 11008]: too large for a full oracle pass to be cheap; checked through properties and a row sample
+    from lingua_amd import ops
+    g = torch.Generator(device="cuda").manual_seed(0)
+    h = torch.randn(16384, 11008, generator=g, device="cuda", dtype=torch.float32).to(torch.bfloat16)
+    col = torch.zeros(11008, dtype=torch.float32, device="cuda")
+    q, s, a = ops.cast_rowwise(h, col_amax=col)
+    qb = q.view(torch.uint8)
+    assert ((qb & 0x7F).amax(dim=1) == 0x7E).all()          # every row reaches +-448
+    assert torch.equal(a.reshape(-1), h.abs().amax(dim=1))
+    assert torch.equal(col, h.abs().amax(dim=0).float())
+    rows = torch.arange(0, 16384, 257)
+    qo, so, _ = oracle.cast_rowwise(h[rows.cuda()].cpu())
+    assert torch.equal(qb[rows.cuda()].cpu(), qo) and bits_equal(s.reshape(-1)[rows.cuda()].cpu(), so)
+    # transposed cast == row-wise cast of the transpose, both on the GPU
+    qt, st = ops.cast_colwise_transposed(h, col)
+    ht = h.t().contiguous()
+    q2, s2, _ = ops.cast_rowwise(ht)
+    assert torch.equal(qt.view(torch.uint8), q2.view(torch.uint8)) and torch.equal(st, s2)

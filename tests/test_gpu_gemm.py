@@ -1,0 +1,129 @@
+"""GPU parity of the fp8 NT GEMM: exact on integer-valued operands (pins the
+matrix-core lane layout, tile edges and K tails), within rel-L2 <= 1e-3 of the
+oracle's bf16(fp32-accumulated dequantised product) on random operands."""
+import pytest
+import torch
+
+import oracle
+from conftest import rel_l2, seeded_bf16
+
+pytestmark = pytest.mark.gpu
+
+TOL = 1e-3  # rel-L2 of bf16 outputs, from the benchmark specification
+
+
+def n_algos():
+    from lingua_amd import ops
+    return len(ops.gemm_algos())
+
+
+def fp8(t):
+    return t.to(torch.float8_e4m3fn)
+
+
+ALGOS = list(range(0, 10))
+SHAPES_EXACT = [(1, 1, 16), (32, 32, 64), (256, 256, 128), (256, 256, 256), (300, 200, 144), (257, 513, 272),
+                (64, 1000, 48), (1000, 24, 208), (512, 768, 240)]
+
+
+@pytest.mark.parametrize("algo", ALGOS)
+def test_exact_small_integer_operands(algo):
+    from lingua_amd import ops
+    if algo > n_algos():
+        pytest.skip("no such tile configuration")
+    g = torch.Generator().manual_seed(100 + algo)
+    for (M, N, K) in SHAPES_EXACT:
+        A = torch.randint(-1, 2, (M, K), generator=g).float()
+        B = torch.randint(-1, 2, (N, K), generator=g).float()
+        sa = torch.tensor([2.0 ** (i % 5 - 2) for i in range(M)]).reshape(M, 1)
+        sb = torch.tensor([2.0 ** (i % 3) for i in range(N)]).reshape(N, 1)
+        out = ops.gemm_nt(fp8(A).cuda(), fp8(B).cuda(), sa.cuda(), sb.cuda(), algo=algo)
+        want = (A.double() @ B.double().t()) * sa.double() * sb.double().t()
+        assert torch.equal(out.cpu().double(), want), (algo, M, N, K)
+
+
+@pytest.mark.parametrize("algo", [0, 1, 3, 5])
+def test_k_indexing_with_one_hot_operands(algo):
+    # B[n] is one-hot at k = pi(n): C[m,n] = A[m, pi(n)] exactly, for any K (tails included)
+    from lingua_amd import ops
+    g = torch.Generator().manual_seed(5)
+    for (M, N, K) in [(96, 400, 400), (130, 1040, 1040), (64, 2064, 2064), (300, 4096, 4096)]:
+        A = torch.randint(-8, 9, (M, K), generator=g).float()
+        pi = torch.randperm(K, generator=g)[:N]
+        B = torch.zeros(N, K)
+        B[torch.arange(N), pi] = 1.0
+        one = torch.ones(1, 1)
+        out = ops.gemm_nt(fp8(A).cuda(), fp8(B).cuda(), one.cuda(), one.cuda(), algo=algo)
+        assert torch.equal(out.cpu().float(), A[:, pi]), (M, N, K)
+        # and the mirrored case: one-hot A picks rows of B
+        out2 = ops.gemm_nt(fp8(B).cuda(), fp8(A).cuda(), one.cuda(), one.cuda(), algo=algo)
+        assert torch.equal(out2.cpu().float(), A[:, pi].t()), (M, N, K)
+
+
+def random_fp8_bytes(shape, g):
+    q = torch.randint(0, 256, shape, generator=g, dtype=torch.int32).to(torch.uint8)
+    q[(q & 0x7F) == 0x7F] = 0x38
+    return q
+
+
+@pytest.mark.parametrize("algo", ALGOS)
+def test_random_operands_vs_oracle(algo):
+    from lingua_amd import ops
+    if algo > n_algos():
+        pytest.skip("no such tile configuration")
+    g = torch.Generator().manual_seed(200 + algo)
+    for (M, N, K) in [(384, 320, 512), (100, 72, 80), (513, 260, 1040)]:
+        qa, qb = random_fp8_bytes((M, K), g), random_fp8_bytes((N, K), g)
+        sa = torch.rand(M, 1, generator=g) + 0.5
+        sb = torch.rand(N, 1, generator=g) + 0.5
+        bias = (torch.randn(N, generator=g) * 50).to(torch.bfloat16)
+        A, B = qa.cuda().view(torch.float8_e4m3fn), qb.cuda().view(torch.float8_e4m3fn)
+        for sa_, sb_, b_ in ((sa, sb, None), (sa, sb, bias), (sa, sb[:1], None), (sa[:1], sb[:1], bias)):
+            out = ops.gemm_nt(A, B, sa_.cuda(), sb_.cuda(), b_.cuda() if b_ is not None else None, algo=algo)
+            want = oracle.gemm_nt(qa, qb, sa_, sb_, b_)
+            assert rel_l2(out, want) <= TOL, (algo, M, N, K)
+
+
+def test_output_leading_dimension_and_unaligned_n():
+    from lingua_amd import ops
+    g = torch.Generator().manual_seed(9)
+    M, N, K = 70, 52, 96
+    qa, qb = random_fp8_bytes((M, K), g), random_fp8_bytes((N, K), g)
+    sa, sb = torch.ones(M, 1), torch.ones(N, 1)
+    buf = torch.full((M, 64), 7.0, dtype=torch.bfloat16, device="cuda")
+    out = buf[:, 4:4 + N]
+    ops.gemm_nt(qa.cuda().view(torch.float8_e4m3fn), qb.cuda().view(torch.float8_e4m3fn), sa.cuda(), sb.cuda(), out=out)
+    want = oracle.gemm_nt(qa, qb, sa, sb)
+    assert rel_l2(out, want) <= TOL
+    assert (buf[:, :4] == 7.0).all() and (buf[:, 4 + N:] == 7.0).all()  # nothing written outside the view
+
+
+def test_config1_forward_product_full_vs_oracle():
+    from lingua_amd import ops
+    x = seeded_bf16((4096, 2048), 1.0, seed=0)
+    w = seeded_bf16((2048, 2048), 0.02, seed=1)
+    qx, sx, _ = ops.cast_rowwise(x.cuda())
+    qw, sw, _ = ops.cast_rowwise(w.cuda())
+    out = ops.gemm_nt(qx, qw, sx, sw)
+    want = oracle.gemm_nt(qx.cpu().view(torch.uint8), qw.cpu().view(torch.uint8), sx.cpu(), sw.cpu())
+    assert rel_l2(out, want) <= TOL
+
+
+@pytest.mark.parametrize("mnk", [(16384, 11008, 4096), (16384, 4096, 11008), (11008, 4096, 16384)])
+def test_7b_shapes_vs_library_matmul_and_oracle_rows(mnk):
+    # full size: against torch's fp32 GPU matmul of the dequantised operands (an independent library routine),
+    # and a sample of rows against the CPU oracle
+    from lingua_amd import ops
+    M, N, K = mnk
+    g = torch.Generator(device="cuda").manual_seed(M + N)
+    a = torch.randn(M, K, generator=g, device="cuda").to(torch.bfloat16)
+    b = (torch.randn(N, K, generator=g, device="cuda") * 0.02).to(torch.bfloat16)
+    qa, sa, _ = ops.cast_rowwise(a)
+    qb, sb, _ = ops.cast_rowwise(b)
+    out = ops.gemm_nt(qa, qb, sa, sb)
+    torch.backends.cuda.matmul.allow_tf32 = False
+    ref = ((qa.float() * sa) @ (qb.float() * sb).t()).to(torch.bfloat16)
+    assert rel_l2(out, ref) <= TOL
+    rows = torch.arange(0, M, max(1, M // 48), device="cuda")[:48]
+    want = oracle.gemm_nt(qa[rows].cpu().view(torch.uint8), qb.cpu().view(torch.uint8), sa[rows].cpu(), sb.cpu())
+    assert rel_l2(out[rows], want) <= TOL

@@ -1,0 +1,199 @@
+"""GPU parity of the drop-in module / autograd function against the oracle's
+three products (forward, dgrad, wgrad) and the reference interface behaviour."""
+import pytest
+import torch
+from torch import nn
+
+import oracle
+from oracle import recipe_torch as rt
+from conftest import rel_l2, seeded_bf16
+from golden_util import load_golden
+
+pytestmark = pytest.mark.gpu
+
+TOL = 1e-3
+
+
+def run_fn(x, w, go, bias=None, x_grad=True, w_grad=True):
+    from lingua_amd.float8 import Fp8LinearFn
+    xd = x.cuda().requires_grad_(x_grad)
+    wd = w.cuda().requires_grad_(w_grad)
+    bd = bias.cuda().requires_grad_(True) if bias is not None else None
+    y = Fp8LinearFn.apply(xd, wd, bd)
+    y.backward(go.cuda())
+    return y.detach(), xd.grad, wd.grad, (bd.grad if bd is not None else None)
+
+
+def test_golden_forward_backward():
+    g = load_golden()
+    y, dx, dw, db = run_fn(g["x_prod"], g["w"], g["go"], g["bias"])
+    assert rel_l2(y, g["y"]) <= TOL
+    assert rel_l2(dx, g["dx"]) <= TOL
+    assert rel_l2(dw, g["dw_fp8"]) <= TOL
+    assert rel_l2(db, g["go"].float().sum(0)) <= 5e-3
+    assert y.dtype == dx.dtype == dw.dtype == torch.bfloat16
+
+
+def test_reference_bf16_wgrad_option():
+    from lingua_amd import float8
+    g = load_golden()
+    float8.config.fp8_wgrad = False
+    try:
+        y, dx, dw, _ = run_fn(g["x_prod"], g["w"], g["go"])
+    finally:
+        float8.config.fp8_wgrad = True
+    assert rel_l2(dw, g["dw_bf16"]) <= 5e-3
+    assert rel_l2(dx, g["dx"]) <= TOL
+
+
+def test_grads_are_none_where_not_required():
+    g = load_golden()
+    _, dx, dw, _ = run_fn(g["x_prod"], g["w"], g["go"], x_grad=False)
+    assert dx is None and rel_l2(dw, g["dw_fp8"]) <= TOL
+    _, dx, dw, _ = run_fn(g["x_prod"], g["w"], g["go"], w_grad=False)
+    assert dw is None and rel_l2(dx, g["dx"]) <= TOL
+
+
+@pytest.mark.parametrize("mkn", [(512, 256, 384), (1000, 272, 136), (2048, 1024, 4096)])
+def test_three_products_vs_oracle(mkn):
+    M, K, N = mkn
+    x = seeded_bf16((M, K), 1.0, seed=1)
+    w = seeded_bf16((N, K), 0.02, seed=2)
+    go = seeded_bf16((M, N), 1e-2, seed=3)
+    y, dx, dw, _ = run_fn(x, w, go)
+    assert rel_l2(y, oracle.linear_forward(x, w)) <= TOL
+    assert rel_l2(dx, oracle.linear_dgrad(go, w)) <= TOL
+    assert rel_l2(dw, oracle.linear_wgrad_fp8(go, x)) <= TOL
+
+
+def test_config1_forward_and_module_surface():
+    from lingua_amd import convert_linears_to_fp8, Fp8Linear
+    x = seeded_bf16((4096, 2048), 1.0, seed=0)
+    w = seeded_bf16((2048, 2048), 0.02, seed=1)
+    lin = nn.Linear(2048, 2048, bias=False, dtype=torch.bfloat16, device="cuda")
+    with torch.no_grad():
+        lin.weight.copy_(w)
+    m = convert_linears_to_fp8(nn.Sequential(lin), "rowwise", "")
+    assert type(m[0]) is Fp8Linear and m[0].weight is lin.weight
+    y = m(x.cuda().reshape(8, 512, 2048))                     # any-rank input: flattened, then restored
+    assert y.shape == (8, 512, 2048) and y.dtype == torch.bfloat16
+    want = oracle.linear_forward(x, w)
+    assert rel_l2(y.reshape(4096, 2048), want) <= TOL
+    # the torch-op restatement agrees too (the figure the benchmark's CPU baseline times)
+    assert rel_l2(y.reshape(4096, 2048), rt.linear_forward(x, w)) <= TOL
+
+
+class SwiGLU(nn.Module):
+    """SwiGLU feed-forward with the layer names of lingua/transformer.py:430-471."""
+
+    def __init__(self, dim, hidden):
+        super().__init__()
+        self.w1 = nn.Linear(dim, hidden, bias=False)
+        self.w3 = nn.Linear(dim, hidden, bias=False)
+        self.w2 = nn.Linear(hidden, dim, bias=False)
+
+    def forward(self, x):
+        return self.w2(torch.nn.functional.silu(self.w1(x)) * self.w3(x))
+
+
+def make_mlp(dim, hidden, seed):
+    from lingua_amd import convert_linears_to_fp8
+    g = torch.Generator().manual_seed(seed)
+    m = SwiGLU(dim, hidden).to(torch.bfloat16)
+    with torch.no_grad():
+        for p in m.parameters():
+            p.copy_((torch.randn(p.shape, generator=g) * 0.02).to(torch.bfloat16))
+    cpu_w = {k: v.detach().clone() for k, v in m.state_dict().items()}
+    layers = nn.ModuleDict({"layers": nn.ModuleList([m])})    # dotted names "layers.0.w1" as the default filter expects
+    layers = convert_linears_to_fp8(layers.cuda(), "rowwise", r"layers\.[0-9]+\.")
+    return layers["layers"][0], cpu_w
+
+
+def test_config2_1b_mlp_forward_rows_vs_oracle():
+    # rows of a row-wise-scaled forward are independent: a sample of token rows pins the full-size result
+    dim, hidden, tokens = 2048, 8192, 32768
+    mlp, w = make_mlp(dim, hidden, seed=0)
+    x = seeded_bf16((tokens, dim), 1.0, seed=0)
+    with torch.no_grad():
+        y = mlp(x.cuda().reshape(8, 4096, dim)).reshape(tokens, dim)
+    rows = torch.arange(0, tokens, tokens // 32)[:32]
+    xs = x[rows]
+    x1 = oracle.linear_forward(xs, w["w1.weight"])
+    x3 = oracle.linear_forward(xs, w["w3.weight"])
+    h = torch.nn.functional.silu(x1) * x3
+    want = oracle.linear_forward(h, w["w2.weight"])
+    assert rel_l2(y[rows.cuda()], want) <= 3 * TOL   # three chained bf16 roundings; each product alone is within TOL
+
+
+def test_config3_7b_mlp_forward_backward():
+    dim, hidden, tokens = 4096, 11008, 16384
+    mlp, w = make_mlp(dim, hidden, seed=0)
+    x = seeded_bf16((tokens, dim), 1.0, seed=0)
+    gy = seeded_bf16((tokens, dim), 1e-2, seed=1)
+    xd = x.cuda().requires_grad_(True)
+    # capture the intermediate activations / gradients the three linears see
+    seen = {}
+    hooks = []
+    for name in ("w1", "w2", "w3"):
+        lin = getattr(mlp, name)
+        hooks.append(lin.register_forward_hook(lambda m_, inp, out, name=name: seen.__setitem__(name + "_in", inp[0].detach())))
+        hooks.append(lin.register_full_backward_hook(lambda m_, gin, gout, name=name: seen.__setitem__(name + "_gout", gout[0].detach())))
+    y = mlp(xd)
+    y.backward(gy.cuda())
+    for h_ in hooks:
+        h_.remove()
+    rows = torch.arange(0, tokens, tokens // 24)[:24]
+    # forward and dgrad of every linear on a row sample (rows are independent)
+    for name in ("w1", "w3", "w2"):
+        W = w[name + ".weight"]
+        a_in = seen[name + "_in"].reshape(tokens, -1)
+        g_out = seen[name + "_gout"].reshape(tokens, -1)
+        lin = getattr(mlp, name)
+        # wgrad on a sample of output rows x input columns (the reduction runs over every token)
+        n_idx = torch.arange(0, W.shape[0], max(1, W.shape[0] // 40))[:40]
+        k_idx = torch.arange(0, W.shape[1], max(1, W.shape[1] // 40))[:40]
+        qg, sg = oracle.cast_colwise_transposed(g_out[:, n_idx.cuda()].cpu())
+        qa, sa = oracle.cast_colwise_transposed(a_in[:, k_idx.cuda()].cpu())
+        want_dw = oracle.gemm_nt(qg, qa, sg, sa)
+        got_dw = lin.weight.grad[n_idx.cuda()][:, k_idx.cuda()]
+        assert rel_l2(got_dw, want_dw) <= TOL, name
+    want_y = None
+    xs = x[rows]
+    x1 = oracle.linear_forward(xs, w["w1.weight"])
+    x3 = oracle.linear_forward(xs, w["w3.weight"])
+    hh = torch.nn.functional.silu(x1) * x3
+    want_y = oracle.linear_forward(hh, w["w2.weight"])
+    assert rel_l2(y.detach()[rows.cuda()], want_y) <= 3 * TOL
+    # dgrad of w2 on the row sample: dh = dgrad(gy, w2)
+    dh_rows = oracle.linear_dgrad(gy[rows], w["w2.weight"])
+    # the GPU's dh is not kept by autograd; recompute it through the function for the same rows
+    from lingua_amd.float8 import Fp8LinearFn
+    hd = hh.cuda().requires_grad_(True)
+    Fp8LinearFn.apply(hd, mlp.w2.weight.detach(), None).backward(gy[rows].cuda())
+    assert rel_l2(hd.grad, dh_rows) <= TOL
+    assert xd.grad is not None and xd.grad.shape == x.shape and torch.isfinite(xd.grad.float()).all()
+
+
+def test_outlier_stress_rowwise_beats_tensorwise_on_the_linear():
+    # config 4: same 4096 -> 11008 linear, row-wise vs tensor-wise scaling of x and W
+    from lingua_amd import ops
+    from test_gpu_cast import outlier_stress_input
+    x, ch, zr = outlier_stress_input(rows=4096, cols=4096, seed=0)
+    w = seeded_bf16((11008, 4096), 0.02, seed=1)
+    xd, wd = x.cuda(), w.cuda()
+    qx, sx, ax = ops.cast_rowwise(xd)
+    qw, sw, aw = ops.cast_rowwise(wd)
+    y_row = ops.gemm_nt(qx, qw, sx, sw)
+    qxt, sxt = ops.cast_tensorwise(xd, ops.amax_reduce(ax))
+    qwt, swt = ops.cast_tensorwise(wd, ops.amax_reduce(aw))
+    y_ten = ops.gemm_nt(qxt, qwt, sxt, swt)
+    rows = torch.arange(0, 4096, 128)
+    want_row = oracle.gemm_nt(qx[rows.cuda()].cpu().view(torch.uint8), qw.cpu().view(torch.uint8), sx[rows.cuda()].cpu(), sw.cpu())
+    want_ten = oracle.gemm_nt(qxt[rows.cuda()].cpu().view(torch.uint8), qwt.cpu().view(torch.uint8), sxt.cpu(), swt.cpu())
+    assert rel_l2(y_row[rows.cuda()], want_row) <= TOL
+    assert rel_l2(y_ten[rows.cuda()], want_ten) <= TOL
+    exact = (xd.float() @ wd.float().t())
+    e_row = rel_l2(y_row, exact)
+    e_ten = rel_l2(y_ten, exact)
+    assert e_row < e_ten
+    assert (y_row[zr.cuda()] == 0).all()                      # all-zero token rows give exact zeros

@@ -1,0 +1,142 @@
+"""CPU-only checks of the host side: the C ABI exports what the header
+declares, argument validation happens before any launch, and the converter /
+module mirror the reference interface (lingua/float8.py:134-191)."""
+import ctypes
+import os
+import re
+
+import pytest
+import torch
+from torch import nn
+
+import lingua_amd
+from lingua_amd import _lib, ops
+from lingua_amd.float8 import Fp8Linear, convert_linears_to_fp8, named_replace
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def test_library_exports_every_declared_symbol():
+    header = open(os.path.join(ROOT, "include", "lingua_fp8.h")).read()
+    header = re.sub(r"/\*.*?\*/", "", header, flags=re.S)
+    declared = set(re.findall(r"\b(l8_\w+)\s*\(", header))
+    assert {"l8_cast_rowwise", "l8_cast_tensorwise", "l8_cast_colwise_transposed", "l8_gemm_nt", "l8_col_amax",
+            "l8_amax_reduce", "l8_version", "l8_last_error", "l8_device_check"} <= declared
+    lib = ctypes.CDLL(_lib.LIB_PATH)
+    for name in declared:
+        assert hasattr(lib, name), name
+    assert declared == set(_lib.SIGNATURES)
+    assert _lib.load().l8_version() >= 1
+
+
+def test_argument_validation_happens_before_launch():
+    lib = _lib.load()
+    fake = 1 << 20  # never dereferenced: every call below must be rejected on the host
+    assert lib.l8_gemm_nt(fake, fake, 4, 4, 8, 16, 16, fake, 1, fake, 1, None, fake, 4, 0, None) == -1
+    assert "multiple of 16" in _lib.last_error()
+    assert lib.l8_gemm_nt(fake, fake, 4, 4, 16, 16, 16, fake, 7, fake, 1, None, fake, 4, 0, None) == -1
+    assert lib.l8_gemm_nt(fake, fake, 4, 4, 16, 16, 16, fake, 1, fake, 1, None, fake, 4, 99, None) == -1
+    assert lib.l8_gemm_nt(None, fake, 4, 4, 16, 16, 16, fake, 1, fake, 1, None, fake, 4, 0, None) == -1
+    assert lib.l8_gemm_nt(fake + 1, fake, 4, 4, 16, 16, 16, fake, 1, fake, 1, None, fake, 4, 0, None) == -1
+    assert lib.l8_cast_rowwise(fake, 4, 12, 12, fake, 12, fake, None, None, None) == -1
+    assert lib.l8_cast_rowwise(fake, -1, 8, 8, fake, 8, fake, None, None, None) == -1
+    assert lib.l8_cast_tensorwise(fake, 4, 8, 8, None, 0, fake, 8, fake, None) == -1
+    assert lib.l8_cast_colwise_transposed(fake, 4, 8, 8, None, fake, 4, fake, None) == -1
+    # empty problems are accepted and do nothing
+    assert lib.l8_cast_rowwise(None, 0, 8, 8, None, 8, None, None, None, None) == 0
+    assert lib.l8_gemm_nt(None, None, 0, 4, 16, 16, 16, None, 1, None, 1, None, None, 4, 0, None) == 0
+
+
+def test_no_cpu_path():
+    x = torch.zeros(4, 16, dtype=torch.bfloat16)
+    with pytest.raises(RuntimeError, match="no CPU path"):
+        ops.cast_rowwise(x)
+    lin = Fp8Linear(16, 8, bias=False, dtype=torch.bfloat16)
+    with pytest.raises(RuntimeError):
+        lin(x)
+
+
+class Block(nn.Module):
+    def __init__(self):
+        super().__init__()
+        self.w1 = nn.Linear(8, 16, bias=False)
+        self.w2 = nn.Linear(16, 8, bias=True)
+        self.norm = nn.LayerNorm(8)
+
+
+class Model(nn.Module):
+    def __init__(self):
+        super().__init__()
+        self.tok_embeddings = nn.Embedding(10, 8)
+        self.layers = nn.ModuleList([Block(), Block()])
+        self.output = nn.Linear(8, 10, bias=False)
+
+
+def test_unknown_recipe_raises_runtime_error():
+    with pytest.raises(RuntimeError, match="Unknown float8 recipe 'tensorwise'"):
+        convert_linears_to_fp8(Model(), "tensorwise", r"layers\.[0-9]+\.")
+
+
+def test_converter_filter_identity_and_state_dict():
+    with torch.device("meta"):
+        m = Model()
+    params_before = dict(m.named_parameters())
+    keys_before = list(m.state_dict().keys())
+    out = convert_linears_to_fp8(m, "rowwise", r"layers\.[0-9]+\.")
+    assert out is m
+    for i in range(2):
+        for name in ("w1", "w2"):
+            lin = getattr(m.layers[i], name)
+            assert type(lin) is Fp8Linear and isinstance(lin, nn.Linear)
+            assert lin.weight is params_before[f"layers.{i}.{name}.weight"]
+            assert lin.weight.device.type == "meta"
+        assert m.layers[i].w2.bias is params_before[f"layers.{i}.w2.bias"]
+        assert m.layers[i].w1.bias is None
+        assert type(m.layers[i].norm) is nn.LayerNorm
+    assert type(m.output) is nn.Linear                       # excluded by the default filter
+    assert type(m.tok_embeddings) is nn.Embedding
+    assert list(m.state_dict().keys()) == keys_before
+    assert {id(p) for p in m.parameters()} == {id(p) for p in params_before.values()}
+
+
+def test_converting_twice_or_a_subclass_asserts():
+    m = convert_linears_to_fp8(Model(), "rowwise", r"layers\.")
+    with pytest.raises(AssertionError):
+        convert_linears_to_fp8(m, "rowwise", r"layers\.")
+
+    class MyLinear(nn.Linear):
+        pass
+
+    m2 = nn.Sequential(MyLinear(4, 4))
+    with pytest.raises(AssertionError, match="MyLinear"):
+        convert_linears_to_fp8(m2, "rowwise", "")
+    # a subclass that the filter does not match is left alone
+    assert convert_linears_to_fp8(m2, "rowwise", "nomatch") is m2
+
+
+def test_root_linear_is_replaced_and_returned():
+    lin = nn.Linear(8, 4, bias=True, dtype=torch.bfloat16)
+    out = convert_linears_to_fp8(lin, "rowwise", "")
+    assert type(out) is Fp8Linear and out is not lin
+    assert out.weight is lin.weight and out.bias is lin.bias
+    assert out.weight.dtype == torch.bfloat16 and (out.in_features, out.out_features) == (8, 4)
+
+
+def test_named_replace_is_post_order_with_dotted_names():
+    seen = []
+
+    def fn(mod, name):
+        seen.append(name)
+        return mod
+
+    m = Model()
+    assert named_replace(fn, m) is m
+    assert seen[-1] == ""
+    assert seen.index("layers.0.w1") < seen.index("layers.0") < seen.index("layers")
+    assert "layers.1.norm" in seen and "output" in seen
+
+
+def test_public_names_match_reference_module():
+    for name in ("EPS", "scale", "matmul", "Fp8LinearFn", "Fp8Linear", "named_replace", "convert_linears_to_fp8"):
+        assert hasattr(lingua_amd, name)
+    assert lingua_amd.EPS == 1e-12
