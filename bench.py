@@ -1,0 +1,191 @@
+#!/usr/bin/env python3
+"""Benchmark of the fp8 row-wise linear path on one MI355X.
+
+Workload (the configuration the headline metric is quoted on): Llama-7B-shaped
+SwiGLU MLP, dim 4096, ffn 11008, 16384 tokens, forward + backward with every
+linear in row-wise fp8 (forward, dgrad and wgrad on the fp8 matrix cores),
+through the drop-in module API.  One "step" is one forward + backward of the
+MLP = 9 GEMMs of 2*16384*4096*11008 flop = 13 297 218 748 416 flop.
+
+Prints ONE JSON line.  `value` is TFLOP/s over whole steps (casts, SiLU and
+autograd bookkeeping included) with inputs resident in HBM.  `roofline` is the
+GEMM kernel alone, timed with events on its stream inside the timed steps.
+`cpu_baseline` is the same recipe as PyTorch CPU ops on a token sample.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+DIM, FFN, TOKENS = 4096, 11008, 16384
+STEP_FLOP = 18 * TOKENS * DIM * FFN          # 9 GEMMs x 2*M*N*K
+PEAK_FP8_TFLOPS = 5000.0                     # MI355X dense fp8 MFMA, published
+PEAK_HBM_GBPS = 8000.0                       # MI355X HBM3E, published
+
+
+def parse():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--algo", type=int, default=0, help="GEMM tile configuration (0 = library default)")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--cpu-sample-tokens", type=int, default=2048)
+    ap.add_argument("--no-kernel-timing", action="store_true", help="do not record per-kernel events in the timed steps")
+    return ap.parse_args()
+
+
+def make_mlp(torch, nn, dim, ffn, device):
+    class SwiGLU(nn.Module):
+        # layer names of lingua/transformer.py:430-471
+        def __init__(self):
+            super().__init__()
+            self.w1 = nn.Linear(dim, ffn, bias=False)
+            self.w3 = nn.Linear(dim, ffn, bias=False)
+            self.w2 = nn.Linear(ffn, dim, bias=False)
+
+        def forward(self, x):
+            return self.w2(torch.nn.functional.silu(self.w1(x)) * self.w3(x))
+
+    g = torch.Generator().manual_seed(0)
+    m = SwiGLU().to(torch.bfloat16)
+    with torch.no_grad():
+        for p in m.parameters():
+            p.copy_((torch.randn(p.shape, generator=g) * 0.02).to(torch.bfloat16))
+    return m.to(device)
+
+
+def cpu_baseline(torch, sample_tokens):
+    """The recipe as PyTorch CPU ops (oracle/recipe_torch.py), on `sample_tokens` tokens of the same workload."""
+    from oracle import recipe_torch as rt
+    cores = os.cpu_count() or 1
+    try:
+        cores = len(os.sched_getaffinity(0))
+    except Exception:
+        pass
+    cores = min(cores, int(os.environ.get("OMP_NUM_THREADS", cores)))
+    torch.set_num_threads(cores)
+    g = torch.Generator().manual_seed(0)
+    x = torch.randn(sample_tokens, DIM, generator=g).to(torch.bfloat16)
+    gy = (torch.randn(sample_tokens, DIM, generator=g) * 1e-2).to(torch.bfloat16)
+    w1 = (torch.randn(FFN, DIM, generator=g) * 0.02).to(torch.bfloat16)
+    w3 = (torch.randn(FFN, DIM, generator=g) * 0.02).to(torch.bfloat16)
+    w2 = (torch.randn(DIM, FFN, generator=g) * 0.02).to(torch.bfloat16)
+    t0 = time.perf_counter()
+    rt.swiglu_mlp_fwd_bwd(x, w1, w2, w3, gy)
+    dt = time.perf_counter() - t0
+    flop = 18 * sample_tokens * DIM * FFN
+    return {
+        "value": round(flop / dt / 1e12, 4),
+        "unit": "TFLOP/s",
+        "cores": torch.get_num_threads(),
+        "kind": "port",
+        "sample": f"same MLP fwd+bwd on {sample_tokens} of {TOKENS} tokens, one repetition, {dt:.2f} s "
+                  f"(PyTorch CPU ops: amax/clamp/div/reciprocal/mul/to(float8_e4m3fn), dequantise, fp32 matmul, bf16)",
+    }
+
+
+def main():
+    args = parse()
+    if args.gpus != 1:
+        print("bench.py: this build runs on exactly one GPU (no collectives are part of the fp8 linear path); "
+              "use --gpus 1", file=sys.stderr)
+        sys.exit(2)
+    import torch
+    from torch import nn
+    from lingua_amd import convert_linears_to_fp8, ops
+    from lingua_amd import float8 as f8
+
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible", file=sys.stderr)
+        sys.exit(1)
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    f8.config.gemm_algo = args.algo
+
+    mlp = make_mlp(torch, nn, DIM, FFN, dev)
+    model = convert_linears_to_fp8(nn.ModuleDict({"layers": nn.ModuleList([mlp])}), "rowwise", r"layers\.[0-9]+\.")
+    mlp = model["layers"][0]
+    g = torch.Generator().manual_seed(1)
+    x = torch.randn(TOKENS, DIM, generator=g).to(torch.bfloat16).to(dev).requires_grad_(True)
+    gy = (torch.randn(TOKENS, DIM, generator=g) * 1e-2).to(torch.bfloat16).to(dev)
+
+    def step():
+        for p in mlp.parameters():
+            p.grad = None
+        x.grad = None
+        y = mlp(x)
+        y.backward(gy)
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+
+    records = None if args.no_kernel_timing else []
+    ops.kernel_timer = records
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    dt = time.perf_counter() - t0
+    ops.kernel_timer = None
+
+    ms_per_step = dt / args.steps * 1e3
+    tflops = STEP_FLOP / (dt / args.steps) / 1e12
+
+    roofline = None
+    kernels = {}
+    if records:
+        agg = {}
+        for name, e0, e1, work in records:
+            ms = e0.elapsed_time(e1)
+            a = agg.setdefault(name, [0, 0.0, 0])
+            a[0] += 1
+            a[1] += ms
+            a[2] += work
+        for name, (n, ms, work) in agg.items():
+            if name == "gemm_nt":
+                kernels[name] = {"launches": n, "avg_ms": round(ms / n, 4), "TFLOP/s": round(work / (ms * 1e-3) / 1e12, 1)}
+            else:
+                gbps = work / (ms * 1e-3) / 1e9
+                kernels[name] = {"launches": n, "avg_ms": round(ms / n, 4), "GB/s": round(gbps, 1),
+                                 "frac_hbm": round(gbps / PEAK_HBM_GBPS, 4)}
+        n, ms, work = agg["gemm_nt"]
+        achieved = work / (ms * 1e-3) / 1e12
+        roofline = {"kernel": "gemm_nt_kernel (fp8 e4m3 NT GEMM, 2*16384*4096*11008 flop per launch)",
+                    "bound": "mfma", "achieved": round(achieved, 1), "peak": PEAK_FP8_TFLOPS, "unit": "TFLOP/s",
+                    "frac": round(achieved / PEAK_FP8_TFLOPS, 4), "traffic": None}
+
+    out = {
+        "metric": "fp8 rowwise linear fwd+bwd TFLOP/s at 7B MLP",
+        "value": round(tflops, 2),
+        "unit": "TFLOP/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 4),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "fp8_e4m3fn",
+        "data": "synthetic",
+        "config": {"workload": "llama-7B SwiGLU MLP fwd+bwd, row-wise fp8 (configs[2])", "dim": DIM, "ffn": FFN,
+                   "tokens": TOKENS, "flop_per_step": STEP_FLOP, "gemm_algo": args.algo,
+                   "wgrad": "fp8"},
+        "frac_of_fp8_peak": round(tflops / PEAK_FP8_TFLOPS, 4),
+        "roofline": roofline,
+        "kernels": kernels,
+    }
+    if not args.no_cpu_baseline:
+        out["cpu_baseline"] = cpu_baseline(torch, args.cpu_sample_tokens)
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

@@ -272,7 +272,7 @@ struct Algo {
   X(2, 2, 4, 4, 1, 8)  /* 2: same, alternative LDS swizzle       */ \
   X(2, 4, 4, 2, 0, 8)  /* 3: 256x256, 8 waves, 128x64 wave tiles */ \
   X(2, 4, 4, 2, 1, 8)  /* 4: same, alternative LDS swizzle       */ \
-  X(2, 2, 2, 2, 0, 8)  /* 5: 128x128, 4 waves (small problems)   */ \
+  X(2, 2, 2, 2, 1, 8)  /* 5: 128x128, 4 waves (small problems)   */ \
   X(2, 2, 4, 2, 0, 8)  /* 6: 256x128, 4 waves                    */ \
   X(4, 2, 2, 4, 0, 8)  /* 7: 256x256, 8 waves, 64x128 wave tiles */ \
   X(2, 2, 4, 4, 0, 4)  /* 8: algo 1 with shorter groups          */ \
@@ -303,7 +303,7 @@ static int pick_algo(int64_t M, int64_t N, int64_t K) {
   // large problems: 256x256; problems that would leave most of the chip idle
   // with big tiles: 128x128
   const int64_t big_tiles = ((M + 255) / 256) * ((N + 255) / 256);
-  if (big_tiles >= num_cus()) return 1;
+  if (big_tiles >= num_cus()) return 4;
   return 5;
 }
 

@@ -13,6 +13,30 @@ from . import _lib
 SCALE_SCALAR = 0
 SCALE_ROW = 1
 
+# Optional per-kernel timing: when `kernel_timer` is a list, every launch below
+# appends (kernel name, start event, end event, algorithmic work) where the
+# events are recorded on the stream the kernel runs on.  Work is flop for the
+# GEMM and compulsory bytes for the casts.  None (the default) records nothing.
+kernel_timer = None
+
+
+class _timed:
+    __slots__ = ("name", "work", "dev", "ev")
+
+    def __init__(self, name, work, dev):
+        self.name, self.work, self.dev, self.ev = name, work, dev, None
+
+    def __enter__(self):
+        if kernel_timer is not None:
+            self.ev = (torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True))
+            self.ev[0].record(torch.cuda.current_stream(self.dev))
+
+    def __exit__(self, *exc):
+        if self.ev is not None:
+            self.ev[1].record(torch.cuda.current_stream(self.dev))
+            kernel_timer.append((self.name, self.ev[0], self.ev[1], self.work))
+        return False
+
 
 def _prep(t: torch.Tensor, what: str):
     if not t.is_cuda:
@@ -47,9 +71,10 @@ def cast_rowwise(x: torch.Tensor, col_amax: Optional[torch.Tensor] = None, want_
     amax = torch.empty((R, 1), dtype=torch.bfloat16, device=x.device)
     if col_amax is not None and (col_amax.dtype != torch.float32 or col_amax.numel() != C or not col_amax.is_contiguous()):
         raise RuntimeError("cast_rowwise: col_amax must be a contiguous fp32 tensor with C elements")
-    code = _lib.load().l8_cast_rowwise(
-        x.data_ptr(), R, C, _ld(x), q.data_ptr() if want_q else None, C, scale.data_ptr(), amax.data_ptr(),
-        col_amax.data_ptr() if col_amax is not None else None, st)
+    with _timed("cast_rowwise", R * C * (3 if want_q else 2) + 4 * R + (4 * C if col_amax is not None else 0), x.device):
+        code = _lib.load().l8_cast_rowwise(
+            x.data_ptr(), R, C, _ld(x), q.data_ptr() if want_q else None, C, scale.data_ptr(), amax.data_ptr(),
+            col_amax.data_ptr() if col_amax is not None else None, st)
     _lib.check(code, "l8_cast_rowwise")
     return q, scale, amax
 
@@ -85,23 +110,34 @@ def cast_tensorwise(x: torch.Tensor, amax: torch.Tensor, transpose: bool = False
     R, C = x.shape
     q = torch.empty((C, R) if transpose else (R, C), dtype=torch.float8_e4m3fn, device=x.device)
     scale = torch.empty((1, 1), dtype=torch.float32, device=x.device)
-    code = _lib.load().l8_cast_tensorwise(x.data_ptr(), R, C, _ld(x), amax.data_ptr(), int(transpose),
-                                          q.data_ptr(), max(q.shape[1], 1), scale.data_ptr(), st)
+    with _timed("cast_tensorwise_t" if transpose else "cast_tensorwise", R * C * 3 + 4, x.device):
+        code = _lib.load().l8_cast_tensorwise(x.data_ptr(), R, C, _ld(x), amax.data_ptr(), int(transpose),
+                                              q.data_ptr(), max(q.shape[1], 1), scale.data_ptr(), st)
     _lib.check(code, "l8_cast_tensorwise")
     return q, scale
 
 
-def cast_colwise_transposed(x: torch.Tensor, col_amax_f32: torch.Tensor):
-    """scale(x.t().contiguous(), its row amax): returns (q [C,R] fp8, scale [C,1] fp32)."""
+def cast_colwise_transposed(x: torch.Tensor, col_amax_f32: torch.Tensor, pad_to: int = 16):
+    """scale(x.t().contiguous(), its row amax): returns (q [C,Rp] fp8, scale [C,1] fp32).
+
+    Rp is R rounded up to a multiple of ``pad_to``; the padding columns hold
+    e4m3 zeros, so a product whose reduction runs over them is unchanged (the
+    GEMM needs a reduction length that is a multiple of 16, token counts are
+    arbitrary)."""
     x = _rows_2d(x, torch.bfloat16, "cast_colwise_transposed")
     st = _prep(x, "cast_colwise_transposed")
     R, C = x.shape
     if col_amax_f32.dtype != torch.float32 or col_amax_f32.numel() != C or not col_amax_f32.is_contiguous():
         raise RuntimeError("cast_colwise_transposed: col_amax must be a contiguous fp32 tensor with C elements")
-    q = torch.empty((C, R), dtype=torch.float8_e4m3fn, device=x.device)
+    Rp = (R + pad_to - 1) // pad_to * pad_to
+    if Rp == R:
+        q = torch.empty((C, R), dtype=torch.float8_e4m3fn, device=x.device)
+    else:
+        q = torch.zeros((C, Rp), dtype=torch.uint8, device=x.device).view(torch.float8_e4m3fn)
     scale = torch.empty((C, 1), dtype=torch.float32, device=x.device)
-    code = _lib.load().l8_cast_colwise_transposed(x.data_ptr(), R, C, _ld(x), col_amax_f32.data_ptr(),
-                                                  q.data_ptr(), max(R, 1), scale.data_ptr(), st)
+    with _timed("cast_colwise_t", R * C * 3 + 4 * C, x.device):
+        code = _lib.load().l8_cast_colwise_transposed(x.data_ptr(), R, C, _ld(x), col_amax_f32.data_ptr(),
+                                                      q.data_ptr(), max(Rp, 1), scale.data_ptr(), st)
     _lib.check(code, "l8_cast_colwise_transposed")
     return q, scale
 
@@ -129,9 +165,10 @@ def gemm_nt(qa: torch.Tensor, qb: torch.Tensor, sa: torch.Tensor, sb: torch.Tens
         out = torch.empty((M, N), dtype=torch.bfloat16, device=qa.device)
     elif out.dtype != torch.bfloat16 or out.shape != (M, N) or out.stride(1) != 1:
         raise RuntimeError("gemm_nt: out must be bf16 [M,N] with unit column stride")
-    code = _lib.load().l8_gemm_nt(qa.data_ptr(), qb.data_ptr(), M, N, K, _ld(qa), _ld(qb), sa.data_ptr(), sa_mode,
-                                  sb.data_ptr(), sb_mode, bias.data_ptr() if bias is not None else None,
-                                  out.data_ptr(), _ld(out) if M > 1 else max(N, 1), algo, st)
+    with _timed("gemm_nt", 2 * M * N * K, qa.device):
+        code = _lib.load().l8_gemm_nt(qa.data_ptr(), qb.data_ptr(), M, N, K, _ld(qa), _ld(qb), sa.data_ptr(), sa_mode,
+                                      sb.data_ptr(), sb_mode, bias.data_ptr() if bias is not None else None,
+                                      out.data_ptr(), _ld(out) if M > 1 else max(N, 1), algo, st)
     _lib.check(code, "l8_gemm_nt")
     return out
 

@@ -133,7 +133,10 @@ def test_transposed_kernels_shapes(shape):
     assert bits_equal(ca.cpu(), oracle.col_amax(x).float())
     q, s = ops.cast_colwise_transposed(xd, ca)
     qo, so = oracle.cast_colwise_transposed(x)
-    assert torch.equal(q.cpu().view(torch.uint8), qo) and bits_equal(s.cpu().reshape(-1), so)
+    R = shape[0]
+    assert q.shape[1] % 16 == 0 and q.shape[1] - R < 16
+    assert torch.equal(q.cpu().view(torch.uint8)[:, :R], qo) and bits_equal(s.cpu().reshape(-1), so)
+    assert (q.cpu().view(torch.uint8)[:, R:] == 0).all()      # reduction padding is e4m3 zero
     amax = ops.amax_reduce(ops.cast_rowwise(xd, want_q=False)[2])
     assert bits_equal(amax.cpu().reshape(()), oracle.amax_of_amaxes(oracle.row_amax(x)))
     for tr in (False, True):
@@ -151,7 +154,7 @@ def test_colwise_nonfinite_columns():
     xd = dev(x)
     q, s = ops.cast_colwise_transposed(xd, ops.col_amax(xd))
     qo, so = oracle.cast_colwise_transposed(x)
-    assert fp8_equal_mod_nan_sign(q, qo)
+    assert fp8_equal_mod_nan_sign(q[:, :40], qo)
     s = s.cpu().reshape(-1)
     assert s[5].isinf() and s[9].isnan()
     fin = so.isfinite()
