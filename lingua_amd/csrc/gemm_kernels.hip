@@ -8,13 +8,21 @@
 // tokens).
 //
 // Structure
-//   * workgroup tile BM x BN x 128 bytes of K, WM x WN wavefronts, each owning
-//     TM x TN accumulator tiles of 32x32 (v_mfma_f32_32x32x64_f8f6f4);
-//   * global -> LDS by `buffer_load_dwordx4 ... lds` (no staging registers),
-//     two LDS stages, one barrier per K tile;
-//   * LDS rows are 128 bytes (8 chunks of 16 B); chunk c of row r lives at
-//     position c ^ f(r) so that the 16-byte fragment reads of 32 consecutive
-//     rows spread over all banks; the permutation is applied on the global
+//   * workgroup tile BM x BN, K consumed in tiles of 64 bytes (one
+//     v_mfma_f32_32x32x64_f8f6f4 deep), WM x WN wavefronts, each owning
+//     TM x TN accumulator tiles of 32x32;
+//   * global -> LDS by `buffer_load_dwordx4 ... lds` (no staging registers)
+//     into a ring of NS stages.  Measured round-trip latency of a K tile under
+//     load is well above the matrix-core time of one tile, so NS-1 tiles are
+//     kept in flight; waits are partial (`s_waitcnt vmcnt(n)`), one barrier
+//     per K tile;
+//   * fragments are software-pipelined: right after the barrier that
+//     publishes tile k+1, its fragments are read from LDS into a second
+//     register set while the matrix cores work on tile k from the first;
+//   * LDS rows are 64 bytes (4 chunks of 16 B); chunk c of row r lives at
+//     position c ^ ((r >> 2) & 3): the 16-byte fragment reads of any 16
+//     consecutive rows then cover all 64 banks once (no conflicts, checked
+//     with SQ_LDS_BANK_CONFLICT).  The permutation is applied on the global
 //     address side because the LDS side of a direct load is lane-linear;
 //   * the matrix cores compute the tile transposed (D[n][m]) so that each lane
 //     ends up with 4 consecutive n per accumulator quad; a v_permlane32_swap
@@ -23,6 +31,11 @@
 //   * workgroup -> tile mapping is XCD-aware: the 8 XCDs each get a contiguous
 //     range of a grouped (GROUP_M tall) tile order so that the workgroups
 //     resident on one XCD share A and B panels in that XCD's L2.
+//
+// L8_GEMM_DIAG (compile-time, never set in the shipped build) removes one side
+// of the main loop to attribute stalls: 1 = no global loads after the prologue,
+// 2 = no LDS reads / matrix-core work, 3 = no stores of C, 4 / 5 = as 2 with every workgroup (4) or every XCD (5)
+// loading the same tile (all L2 hits).  Results are wrong by construction.
 #include "l8_common.h"
 
 namespace l8 {
@@ -50,14 +63,41 @@ L8_DEV __amdgpu_buffer_rsrc_t make_rsrc(const void *p, uint32_t bytes) {
 
 constexpr uint32_t kOOB = 0x80000000u;  // voffset that is out of range for every resource below
 
-template <int WM, int WN, int TM, int TN, int SWZ, int GROUP_M>
+#ifndef L8_GEMM_DIAG
+#define L8_GEMM_DIAG 0
+#endif
+
+// s_waitcnt for vmcnt <= n and lgkmcnt == 0 (expcnt untouched)
+#define L8_WAIT_VM_LGKM0(n) \
+  __builtin_amdgcn_s_waitcnt(((n) & 0xF) | (0x7 << 4) | (0x0 << 8) | ((((n) >> 4) & 0x3) << 14))
+
+#if defined(__HIP_DEVICE_COMPILE__)
+// Scheduling recipe for one half trip: N_MMA groups of "one MFMA, then a share
+// of the N_DSR LDS reads (spread over the first N_MMA-2 groups), then one of
+// the N_VMEM global loads".  The group sizes must be literals, hence the recursion.
+template <int N_MMA, int N_DSR, int N_VMEM, int I>
+L8_DEV void interleave_step() {
+  if constexpr (I < N_MMA) {
+    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+    constexpr int slots = N_MMA > 2 ? N_MMA - 2 : 1;
+    constexpr int r0 = (N_DSR * I) / slots, r1 = (N_DSR * (I + 1)) / slots;
+    if constexpr (I < slots && r1 > r0) __builtin_amdgcn_sched_group_barrier(0x100, r1 - r0, 0);
+    if constexpr (I < N_VMEM) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
+    interleave_step<N_MMA, N_DSR, N_VMEM, I + 1>();
+  }
+}
+#endif
+
+template <int WM, int WN, int TM, int TN, int NS, int GROUP_M>
 __global__ __launch_bounds__(WM *WN * 64) void gemm_nt_kernel(const GemmArgs p) {
 #if defined(__HIP_DEVICE_COMPILE__)
-  constexpr int BM = WM * TM * 32, BN = WN * TN * 32, BK = 128;
+  constexpr int BM = WM * TM * 32, BN = WN * TN * 32, BK = 64;
   constexpr int NW = WM * WN;
   constexpr int A_BYTES = BM * BK, B_BYTES = BN * BK, STAGE = A_BYTES + B_BYTES;
-  static_assert((BM / 8) % NW == 0 && (BN / 8) % NW == 0, "tile rows must split evenly over waves");
-  constexpr int NA = BM / 8 / NW, NB = BN / 8 / NW;  // 1 KiB wave loads per stage per wave
+  static_assert((BM / 16) % NW == 0 && (BN / 16) % NW == 0, "tile rows must split evenly over waves");
+  constexpr int NA = BM / 16 / NW, NB = BN / 16 / NW;  // 1 KiB wave loads (16 rows x 64 B) per stage per wave
+  constexpr int LPT = NA + NB;                         // loads per K tile per wave
+  static_assert(NS >= 2 && (NS - 1) * LPT <= 63, "vmcnt is a 6-bit counter");
   extern __shared__ __attribute__((aligned(1024))) uint8_t smem[];
 
   const int lane = threadIdx.x & 63;
@@ -80,10 +120,13 @@ __global__ __launch_bounds__(WM *WN * 64) void gemm_nt_kernel(const GemmArgs p) 
     tile_m = first_m + in_grp % gsz;
     tile_n = in_grp / gsz;
   }
+  if (L8_GEMM_DIAG == 4 || L8_GEMM_DIAG == 5) { tile_m = 0; tile_n = (L8_GEMM_DIAG == 5) ? (int)(blockIdx.x & 7) : 0; }
   const int m0 = tile_m * BM, n0 = tile_n * BN;
 
   // ---- global -> LDS load plan ----
-  const int lrow = lane >> 3, lpos = lane & 7;
+  // lane l of a wave load fills LDS row l/4, position l%4 of a 16-row group
+  const int lrow = lane >> 2, lpos = lane & 3;
+  const int lchunk = lpos ^ ((lrow >> 2) & 3);  // which 16-byte chunk of the row this lane fetches
   const uint8_t *Ablk = p.A + (int64_t)m0 * p.lda;
   const uint8_t *Bblk = p.B + (int64_t)n0 * p.ldb;
   const int64_t a_left = (int64_t)(p.M - m0 - 1) * p.lda + p.K;
@@ -92,56 +135,59 @@ __global__ __launch_bounds__(WM *WN * 64) void gemm_nt_kernel(const GemmArgs p) 
   const __amdgpu_buffer_rsrc_t rsB = make_rsrc(Bblk, b_left < 0x7fffffff ? (uint32_t)b_left : 0x7fffffffu);
 
   uint32_t a_voff[NA], b_voff[NB];
-  uint32_t a_chunk[NA], b_chunk[NB];
 #pragma unroll
   for (int i = 0; i < NA; ++i) {
-    const int g = wave * NA + i, row = g * 8 + lrow;
-    const int chunk = lpos ^ lrow ^ (SWZ ? (g & 1) : 0);
-    a_chunk[i] = chunk * 16;
-    a_voff[i] = (m0 + row < p.M) ? (uint32_t)(row * (int)p.lda + chunk * 16) : kOOB;
+    const int row = (wave * NA + i) * 16 + lrow;
+    a_voff[i] = (m0 + row < p.M) ? (uint32_t)(row * (int)p.lda + lchunk * 16) : kOOB;
   }
 #pragma unroll
   for (int i = 0; i < NB; ++i) {
-    const int g = wave * NB + i, row = g * 8 + lrow;
-    const int chunk = lpos ^ lrow ^ (SWZ ? (g & 1) : 0);
-    b_chunk[i] = chunk * 16;
-    b_voff[i] = (n0 + row < p.N) ? (uint32_t)(row * (int)p.ldb + chunk * 16) : kOOB;
+    const int row = (wave * NB + i) * 16 + lrow;
+    b_voff[i] = (n0 + row < p.N) ? (uint32_t)(row * (int)p.ldb + lchunk * 16) : kOOB;
   }
 
-  auto issue = [&](int stage, int k0) {
+  const int KT = (p.K + BK - 1) / BK;
+  // Every call issues exactly LPT loads so that the vmcnt arithmetic below is
+  // uniform; tiles at or beyond KT, rows beyond M / N and chunks beyond K use
+  // an out-of-range offset, which the buffer unit turns into zeros in LDS.
+  auto issue = [&](int kt) {
+    const int stage = kt % NS;
+    const int k0 = kt * BK;
     uint8_t *sA = smem + stage * STAGE + wave * (NA * 1024);
     uint8_t *sB = smem + stage * STAGE + A_BYTES + wave * (NB * 1024);
-    if (k0 + BK <= p.K) {
+    // per-lane mask: chunks at or beyond K (partial last tile, tiles past the end) go out of range
+    const uint32_t kmask = (k0 + lchunk * 16 < p.K) ? 0u : kOOB;
 #pragma unroll
-      for (int i = 0; i < NA; ++i)
-        __builtin_amdgcn_raw_ptr_buffer_load_lds(rsA, (lds_ptr_t)(sA + i * 1024), 16, a_voff[i], k0, 0, 0);
+    for (int i = 0; i < NA; ++i)
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(rsA, (lds_ptr_t)(sA + i * 1024), 16, a_voff[i] | kmask, k0, 0, 0);
 #pragma unroll
-      for (int i = 0; i < NB; ++i)
-        __builtin_amdgcn_raw_ptr_buffer_load_lds(rsB, (lds_ptr_t)(sB + i * 1024), 16, b_voff[i], k0, 0, 0);
-    } else {  // last, partial K tile: chunks at or beyond K read as zero
-#pragma unroll
-      for (int i = 0; i < NA; ++i) {
-        const uint32_t v = (k0 + (int)a_chunk[i] < p.K) ? a_voff[i] : kOOB;
-        __builtin_amdgcn_raw_ptr_buffer_load_lds(rsA, (lds_ptr_t)(sA + i * 1024), 16, v, k0, 0, 0);
-      }
-#pragma unroll
-      for (int i = 0; i < NB; ++i) {
-        const uint32_t v = (k0 + (int)b_chunk[i] < p.K) ? b_voff[i] : kOOB;
-        __builtin_amdgcn_raw_ptr_buffer_load_lds(rsB, (lds_ptr_t)(sB + i * 1024), 16, v, k0, 0, 0);
-      }
-    }
+    for (int i = 0; i < NB; ++i)
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(rsB, (lds_ptr_t)(sB + i * 1024), 16, b_voff[i] | kmask, k0, 0, 0);
   };
 
   // ---- LDS -> register fragment plan ----
   const int l31 = lane & 31, h = lane >> 5;
-  const int fr = (l31 & 7) ^ (SWZ ? ((l31 >> 3) & 1) : 0);
-  int foff[2][2];
-#pragma unroll
-  for (int s = 0; s < 2; ++s)
-#pragma unroll
-    for (int j = 0; j < 2; ++j) foff[s][j] = l31 * BK + (((s * 4 + h * 2 + j) ^ fr) * 16);
+  const int fr = (l31 >> 2) & 3;
+  const int foff0 = l31 * BK + (((h * 2 + 0) ^ fr) * 16);
+  const int foff1 = l31 * BK + (((h * 2 + 1) ^ fr) * 16);
   const int a_base = wm * (TM * 32 * BK);
   const int b_base = A_BYTES + wn * (TN * 32 * BK);
+
+  auto read_frags = [&](int kt, v8i (&af)[TM], v8i (&bf)[TN]) {
+    const uint8_t *st = smem + (kt % NS) * STAGE;
+#pragma unroll
+    for (int tm = 0; tm < TM; ++tm) {
+      const v4i lo = *(const v4i *)(st + a_base + tm * (32 * BK) + foff0);
+      const v4i hi = *(const v4i *)(st + a_base + tm * (32 * BK) + foff1);
+      af[tm] = v8i{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+    }
+#pragma unroll
+    for (int tn = 0; tn < TN; ++tn) {
+      const v4i lo = *(const v4i *)(st + b_base + tn * (32 * BK) + foff0);
+      const v4i hi = *(const v4i *)(st + b_base + tn * (32 * BK) + foff1);
+      bf[tn] = v8i{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+    }
+  };
 
   v16f acc[TN][TM];
 #pragma unroll
@@ -151,35 +197,74 @@ __global__ __launch_bounds__(WM *WN * 64) void gemm_nt_kernel(const GemmArgs p) 
 #pragma unroll
       for (int v = 0; v < 16; ++v) acc[tn][tm][v] = 0.0f;
 
-  const int KT = (p.K + BK - 1) / BK;
-  issue(0, 0);
-  for (int kt = 0; kt < KT; ++kt) {
-    __syncthreads();  // tile kt has landed for every wave; stage (kt+1)&1 is free
-    if (kt + 1 < KT) issue((kt + 1) & 1, (kt + 1) * BK);
-    const uint8_t *st = smem + (kt & 1) * STAGE;
+  auto mma = [&](v8i (&af)[TM], v8i (&bf)[TN]) {
 #pragma unroll
-    for (int s = 0; s < 2; ++s) {
-      v8i af[TM], bf[TN];
+    for (int tn = 0; tn < TN; ++tn)
 #pragma unroll
-      for (int tm = 0; tm < TM; ++tm) {
-        const v4i lo = *(const v4i *)(st + a_base + tm * (32 * BK) + foff[s][0]);
-        const v4i hi = *(const v4i *)(st + a_base + tm * (32 * BK) + foff[s][1]);
-        af[tm] = v8i{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
-      }
+      for (int tm = 0; tm < TM; ++tm)
+        // D[i = n][j = m]: B rows feed the "A" port, A rows the "B" port
+        acc[tn][tm] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(bf[tn], af[tm], acc[tn][tm], 0, 0, 0, 0, 0, 0);
+  };
+
+  // Ring bookkeeping.  Tile t lives in stage t % NS; each wave issues LPT
+  // loads per tile, in tile order.  At the top of iteration kt the loads of
+  // tiles kt+1 .. kt+NS-1 may be outstanding; waiting until at most
+  // (NS-2)*LPT remain means this wave's part of tile kt+1 has landed, and the
+  // barrier extends that to every wave.  The same wait also drains this wave's
+  // LDS reads of tile kt (lgkmcnt 0), so after the barrier every wave holds
+  // tile kt in registers and stage kt % NS can be refilled with tile kt+NS.
+  // The empty asm statements keep the compiler from moving LDS accesses across.
+#define L8_PUBLISH_NEXT()                  \
+  do {                                     \
+    L8_WAIT_VM_LGKM0((NS - 2) * LPT);      \
+    asm volatile("" ::: "memory");         \
+    __builtin_amdgcn_s_barrier();          \
+    asm volatile("" ::: "memory");         \
+  } while (0)
+
+  // prologue: all NS stages in flight, tile 0 published and read
 #pragma unroll
-      for (int tn = 0; tn < TN; ++tn) {
-        const v4i lo = *(const v4i *)(st + b_base + tn * (32 * BK) + foff[s][0]);
-        const v4i hi = *(const v4i *)(st + b_base + tn * (32 * BK) + foff[s][1]);
-        bf[tn] = v8i{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
-      }
-#pragma unroll
-      for (int tn = 0; tn < TN; ++tn)
-#pragma unroll
-        for (int tm = 0; tm < TM; ++tm)
-          // D[i = n][j = m]: B rows feed the "A" port, A rows the "B" port
-          acc[tn][tm] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(bf[tn], af[tm], acc[tn][tm], 0, 0, 0, 0, 0, 0);
+  for (int t = 0; t < NS; ++t) issue(t);
+  v8i af0[TM], bf0[TN], af1[TM], bf1[TN];
+  L8_WAIT_VM_LGKM0((NS - 1) * LPT);
+  asm volatile("" ::: "memory");
+  __builtin_amdgcn_s_barrier();
+  asm volatile("" ::: "memory");
+  read_frags(0, af0, bf0);
+
+  // Issue order inside one half trip.  A wave issues in order, and right after
+  // the barrier all waves push their LDS reads at once; if those came first,
+  // each wave's matrix-core work would wait behind the whole backlog.  So the
+  // reads (and the global loads) are spread between the MFMAs, which need
+  // nothing but registers that are already valid.
+  constexpr int N_MMA = TM * TN, N_DSR = 2 * (TM + TN);
+  auto interleave = [&]() { interleave_step<N_MMA, N_DSR, (L8_GEMM_DIAG == 1 ? 0 : LPT), 0>(); };
+
+  // Two tiles per trip so that the two fragment sets keep fixed registers.  An
+  // odd tile count is rounded up: the extra tile was loaded out of range, i.e.
+  // as zeros, and adds nothing.
+  for (int kt = 0; kt < KT; kt += 2) {
+    // matrix cores on tile kt (set 0) while tile kt+1 is read into set 1
+    L8_PUBLISH_NEXT();
+    if (L8_GEMM_DIAG != 1) issue(kt + NS);
+    if (L8_GEMM_DIAG != 2 && L8_GEMM_DIAG != 4 && L8_GEMM_DIAG != 5) {
+      read_frags(kt + 1, af1, bf1);
+      mma(af0, bf0);
+      interleave();
     }
+    __builtin_amdgcn_sched_barrier(0);
+    // matrix cores on tile kt+1 (set 1) while tile kt+2 is read into set 0
+    L8_PUBLISH_NEXT();
+    if (L8_GEMM_DIAG != 1) issue(kt + 1 + NS);
+    if (L8_GEMM_DIAG != 2 && L8_GEMM_DIAG != 4 && L8_GEMM_DIAG != 5) {
+      read_frags(kt + 2, af0, bf0);
+      mma(af1, bf1);
+      interleave();
+    }
+    __builtin_amdgcn_sched_barrier(0);
   }
+  // drain the tail loads (out of range, zero-filling) before LDS is released
+  L8_WAIT_VM_LGKM0(0);
 
   // ---- epilogue ----
   // lane (l31, h) of tile (tn, tm) holds m = l31 and, in accumulator quad qd,
@@ -237,7 +322,7 @@ __global__ __launch_bounds__(WM *WN * 64) void gemm_nt_kernel(const GemmArgs p) 
       // lower lanes: pk[0,1]=n0..3 pk[4,5]=n4..7 pk[2,3]=n8..11 pk[6,7]=n12..15
       // upper lanes: pk[0,1]=n16..19 pk[4,5]=n20..23 pk[2,3]=n24..27 pk[6,7]=n28..31
       const int nbase = nt0 + 16 * h;
-      if (m_okv[tm]) {
+      if (m_okv[tm] && (L8_GEMM_DIAG != 3 || pk[0] == 0x12345678u)) {
         uint16_t *dst = p.C + (int64_t)m * p.ldc + nbase;
         if (c_vec && nbase + 16 <= p.N) {
           *(v4i *)dst = v4i{(int)pk[0], (int)pk[1], (int)pk[4], (int)pk[5]};
@@ -266,25 +351,25 @@ struct Algo {
   int bm, bn, threads, lds;
 };
 
-// X(WM, WN, TM, TN, SWZ, GROUP_M) -- 1-based position in this list is the `algo` number
-#define L8_ALGO_LIST(X)                                             \
-  X(2, 2, 4, 4, 0, 8)  /* 1: 256x256, 4 waves                    */ \
-  X(2, 2, 4, 4, 1, 8)  /* 2: same, alternative LDS swizzle       */ \
-  X(2, 4, 4, 2, 0, 8)  /* 3: 256x256, 8 waves, 128x64 wave tiles */ \
-  X(2, 4, 4, 2, 1, 8)  /* 4: same, alternative LDS swizzle       */ \
-  X(2, 2, 2, 2, 1, 8)  /* 5: 128x128, 4 waves (small problems)   */ \
-  X(2, 2, 4, 2, 0, 8)  /* 6: 256x128, 4 waves                    */ \
-  X(4, 2, 2, 4, 0, 8)  /* 7: 256x256, 8 waves, 64x128 wave tiles */ \
-  X(2, 2, 4, 4, 0, 4)  /* 8: algo 1 with shorter groups          */ \
-  X(2, 2, 4, 4, 0, 16) /* 9: algo 1 with taller groups           */
+// X(WM, WN, TM, TN, NS, GROUP_M) -- 1-based position in this list is the `algo` number
+#define L8_ALGO_LIST(X)                                                      \
+  X(2, 4, 4, 2, 4, 8)  /* 1: 256x256, 8 waves (128x64 each), 4 stages     */ \
+  X(2, 4, 4, 2, 5, 8)  /* 2: same, 5 stages (all 160 KiB of LDS)          */ \
+  X(2, 2, 4, 4, 4, 8)  /* 3: 256x256, 4 waves (128x128 each), 4 stages    */ \
+  X(2, 2, 4, 4, 5, 8)  /* 4: same, 5 stages                               */ \
+  X(2, 2, 2, 2, 4, 8)  /* 5: 128x128, 4 waves (small problems)            */ \
+  X(4, 2, 2, 4, 4, 8)  /* 6: 256x256, 8 waves (64x128 each), 4 stages     */ \
+  X(2, 4, 4, 2, 3, 8)  /* 7: algo 1 with 3 stages                         */ \
+  X(2, 4, 4, 2, 4, 4)  /* 8: algo 1 with shorter groups                   */ \
+  X(2, 4, 4, 2, 4, 16) /* 9: algo 1 with taller groups                    */
 
-#define L8_INSTANTIATE(WM, WN, TM, TN, SWZ, GM) \
-  template __global__ void gemm_nt_kernel<WM, WN, TM, TN, SWZ, GM>(const GemmArgs);
+#define L8_INSTANTIATE(WM, WN, TM, TN, NS, GM) \
+  template __global__ void gemm_nt_kernel<WM, WN, TM, TN, NS, GM>(const GemmArgs);
 L8_ALGO_LIST(L8_INSTANTIATE)
 
-#define L8_ALGO_ROW(WM, WN, TM, TN, SWZ, GM)                                                          \
-  {"mt" #WM "x" #WN "w_" #TM "x" #TN "t_swz" #SWZ "_g" #GM, gemm_nt_kernel<WM, WN, TM, TN, SWZ, GM>, \
-   WM * TM * 32, WN * TN * 32, WM * WN * 64, 2 * (WM * TM * 32 + WN * TN * 32) * 128},
+#define L8_ALGO_ROW(WM, WN, TM, TN, NS, GM)                                                        \
+  {"mt" #WM "x" #WN "w_" #TM "x" #TN "t_ns" #NS "_g" #GM, gemm_nt_kernel<WM, WN, TM, TN, NS, GM>, \
+   WM * TM * 32, WN * TN * 32, WM * WN * 64, NS * (WM * TM * 32 + WN * TN * 32) * 64},
 
 static const Algo kAlgos[] = {L8_ALGO_LIST(L8_ALGO_ROW)};
 constexpr int kNumAlgos = sizeof(kAlgos) / sizeof(kAlgos[0]);
@@ -303,7 +388,7 @@ static int pick_algo(int64_t M, int64_t N, int64_t K) {
   // large problems: 256x256; problems that would leave most of the chip idle
   // with big tiles: 128x128
   const int64_t big_tiles = ((M + 255) / 256) * ((N + 255) / 256);
-  if (big_tiles >= num_cus()) return 4;
+  if (big_tiles >= num_cus()) return 1;
   return 5;
 }
 
