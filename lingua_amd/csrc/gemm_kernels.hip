@@ -8,22 +8,27 @@
 // tokens).
 //
 // Structure
-//   * workgroup tile BM x BN, K consumed in tiles of 64 bytes (one
-//     v_mfma_f32_32x32x64_f8f6f4 deep), WM x WN wavefronts, each owning
+//   * workgroup tile BM x BN, K consumed in tiles of 128 bytes (two
+//     v_mfma_f32_32x32x64_f8f6f4 steps), WM x WN wavefronts, each owning
 //     TM x TN accumulator tiles of 32x32;
-//   * global -> LDS by `buffer_load_dwordx4 ... lds` (no staging registers)
-//     into a ring of NS stages.  Measured round-trip latency of a K tile under
-//     load is well above the matrix-core time of one tile, so NS-1 tiles are
-//     kept in flight; waits are partial (`s_waitcnt vmcnt(n)`), one barrier
-//     per K tile;
-//   * fragments are software-pipelined: right after the barrier that
-//     publishes tile k+1, its fragments are read from LDS into a second
-//     register set while the matrix cores work on tile k from the first;
-//   * LDS rows are 64 bytes (4 chunks of 16 B); chunk c of row r lives at
-//     position c ^ ((r >> 2) & 3): the 16-byte fragment reads of any 16
-//     consecutive rows then cover all 64 banks once (no conflicts, checked
-//     with SQ_LDS_BANK_CONFLICT).  The permutation is applied on the global
-//     address side because the LDS side of a direct load is lane-linear;
+//   * global -> LDS by `buffer_load_dwordx4 ... lds` (no staging registers).
+//     Each row segment is a full 128-byte line: 64-byte segments halve the
+//     L2 request rate that can be sustained (measured).  LDS is a ring of R
+//     slots, each holding the A or the B panel of one K tile; units are
+//     issued in the order A(0), B(0), A(1), ...  With R = 5 the ring holds the
+//     K tile being read, the K tile being published and one more unit, so
+//     loads stay in flight across every barrier; waits are partial
+//     (`s_waitcnt vmcnt(n)`), one barrier per K tile;
+//   * fragments are software-pipelined through two register sets: each half
+//     of a trip runs the MFMAs of one 64-byte step while the next step is
+//     read from LDS, and the instruction order interleaves MFMAs, LDS reads
+//     and global loads (a wave issues in order);
+//   * LDS rows are 128 bytes (8 chunks of 16 B); chunk c of row r lives at
+//     position c ^ f(r), f(r) = (r & 7) ^ ((r >> 3) & 1): the 16-byte
+//     fragment reads of any 16 consecutive rows then cover all 64 banks once
+//     (SQ_LDS_BANK_CONFLICT = 0; f(r) = r & 7 alone measured 50 % conflict
+//     cycles).  The permutation is applied on the global address side because
+//     the LDS side of a direct load is lane-linear;
 //   * the matrix cores compute the tile transposed (D[n][m]) so that each lane
 //     ends up with 4 consecutive n per accumulator quad; a v_permlane32_swap
 //     pairs lanes l / l+32 into 16 consecutive n, scaled, rounded to bf16 and
@@ -34,8 +39,8 @@
 //
 // L8_GEMM_DIAG (compile-time, never set in the shipped build) removes one side
 // of the main loop to attribute stalls: 1 = no global loads after the prologue,
-// 2 = no LDS reads / matrix-core work, 3 = no stores of C, 4 / 5 = as 2 with every workgroup (4) or every XCD (5)
-// loading the same tile (all L2 hits).  Results are wrong by construction.
+// 2 = no LDS reads / matrix-core work, 3 = no stores of C, 4 = as 2 with every workgroup loading the same tile (all
+// L2 hits).  Results are wrong by construction.
 #include "l8_common.h"
 
 namespace l8 {
@@ -88,16 +93,21 @@ L8_DEV void interleave_step() {
 }
 #endif
 
-template <int WM, int WN, int TM, int TN, int NS, int GROUP_M>
+template <int WM, int WN, int TM, int TN, int R, int GROUP_M>
 __global__ __launch_bounds__(WM *WN * 64) void gemm_nt_kernel(const GemmArgs p) {
 #if defined(__HIP_DEVICE_COMPILE__)
-  constexpr int BM = WM * TM * 32, BN = WN * TN * 32, BK = 64;
+  constexpr int BM = WM * TM * 32, BN = WN * TN * 32, BK = 128;
   constexpr int NW = WM * WN;
-  constexpr int A_BYTES = BM * BK, B_BYTES = BN * BK, STAGE = A_BYTES + B_BYTES;
-  static_assert((BM / 16) % NW == 0 && (BN / 16) % NW == 0, "tile rows must split evenly over waves");
-  constexpr int NA = BM / 16 / NW, NB = BN / 16 / NW;  // 1 KiB wave loads (16 rows x 64 B) per stage per wave
-  constexpr int LPT = NA + NB;                         // loads per K tile per wave
-  static_assert(NS >= 2 && (NS - 1) * LPT <= 63, "vmcnt is a 6-bit counter");
+  constexpr int A_BYTES = BM * BK, B_BYTES = BN * BK;
+  constexpr int UNIT = A_BYTES > B_BYTES ? A_BYTES : B_BYTES;  // one ring slot holds an A or a B panel of one K tile
+  static_assert((BM / 8) % NW == 0 && (BN / 8) % NW == 0, "tile rows must split evenly over waves");
+  constexpr int NA = BM / 8 / NW, NB = BN / 8 / NW;  // 1 KiB wave loads (8 rows x 128 B) per panel per wave
+  // loads of the units that may still be in flight when a K tile is published:
+  // the ring holds the tile being read (2 slots), the tile being published (2
+  // slots) and R-4 younger units, the first of which is an A panel
+  constexpr int PEND = ((R - 4 + 1) / 2) * NA + ((R - 4) / 2) * NB;
+  constexpr int PEND0 = ((R - 2 + 1) / 2) * NA + ((R - 2) / 2) * NB;  // same for the prologue (R-2 younger units)
+  static_assert(R >= 4 && PEND0 <= 63, "vmcnt is a 6-bit counter");
   extern __shared__ __attribute__((aligned(1024))) uint8_t smem[];
 
   const int lane = threadIdx.x & 63;
@@ -120,13 +130,13 @@ __global__ __launch_bounds__(WM *WN * 64) void gemm_nt_kernel(const GemmArgs p) 
     tile_m = first_m + in_grp % gsz;
     tile_n = in_grp / gsz;
   }
-  if (L8_GEMM_DIAG == 4 || L8_GEMM_DIAG == 5) { tile_m = 0; tile_n = (L8_GEMM_DIAG == 5) ? (int)(blockIdx.x & 7) : 0; }
+  if (L8_GEMM_DIAG == 4) { tile_m = 0; tile_n = 0; }
   const int m0 = tile_m * BM, n0 = tile_n * BN;
 
   // ---- global -> LDS load plan ----
-  // lane l of a wave load fills LDS row l/4, position l%4 of a 16-row group
-  const int lrow = lane >> 2, lpos = lane & 3;
-  const int lchunk = lpos ^ ((lrow >> 2) & 3);  // which 16-byte chunk of the row this lane fetches
+  // lane l of a wave load fills LDS row l/8, position l%8 of an 8-row group;
+  // position p of row r holds chunk p ^ f(r), f(r) = (r & 7) ^ ((r >> 3) & 1)
+  const int lrow = lane >> 3, lpos = lane & 7;
   const uint8_t *Ablk = p.A + (int64_t)m0 * p.lda;
   const uint8_t *Bblk = p.B + (int64_t)n0 * p.ldb;
   const int64_t a_left = (int64_t)(p.M - m0 - 1) * p.lda + p.K;
@@ -137,54 +147,71 @@ __global__ __launch_bounds__(WM *WN * 64) void gemm_nt_kernel(const GemmArgs p) 
   uint32_t a_voff[NA], b_voff[NB];
 #pragma unroll
   for (int i = 0; i < NA; ++i) {
-    const int row = (wave * NA + i) * 16 + lrow;
-    a_voff[i] = (m0 + row < p.M) ? (uint32_t)(row * (int)p.lda + lchunk * 16) : kOOB;
+    const int g = wave * NA + i, row = g * 8 + lrow;
+    const int chunk = lpos ^ lrow ^ (g & 1);
+    a_voff[i] = (m0 + row < p.M) ? (uint32_t)(row * (int)p.lda + chunk * 16) : kOOB;
   }
 #pragma unroll
   for (int i = 0; i < NB; ++i) {
-    const int row = (wave * NB + i) * 16 + lrow;
-    b_voff[i] = (n0 + row < p.N) ? (uint32_t)(row * (int)p.ldb + lchunk * 16) : kOOB;
+    const int g = wave * NB + i, row = g * 8 + lrow;
+    const int chunk = lpos ^ lrow ^ (g & 1);
+    b_voff[i] = (n0 + row < p.N) ? (uint32_t)(row * (int)p.ldb + chunk * 16) : kOOB;
   }
+  const int chunk_even = (lpos ^ lrow) * 16, chunk_odd = (lpos ^ lrow ^ 1) * 16;  // byte offset in the row, by parity of g
 
   const int KT = (p.K + BK - 1) / BK;
-  // Every call issues exactly LPT loads so that the vmcnt arithmetic below is
-  // uniform; tiles at or beyond KT, rows beyond M / N and chunks beyond K use
-  // an out-of-range offset, which the buffer unit turns into zeros in LDS.
-  auto issue = [&](int kt) {
-    const int stage = kt % NS;
+  // Units are issued in the order A(0), B(0), A(1), B(1), ...; unit u lives in
+  // ring slot u % R.  Every call issues the full count of loads so that the
+  // vmcnt arithmetic is uniform; K tiles at or beyond the end, rows beyond
+  // M / N and chunks beyond K use an out-of-range offset, which the buffer unit
+  // turns into zeros in LDS.
+  auto issue_a = [&](int kt) {
     const int k0 = kt * BK;
-    uint8_t *sA = smem + stage * STAGE + wave * (NA * 1024);
-    uint8_t *sB = smem + stage * STAGE + A_BYTES + wave * (NB * 1024);
-    // per-lane mask: chunks at or beyond K (partial last tile, tiles past the end) go out of range
-    const uint32_t kmask = (k0 + lchunk * 16 < p.K) ? 0u : kOOB;
+    uint8_t *dst = smem + ((2 * kt) % R) * UNIT + wave * (NA * 1024);
+    const uint32_t m_even = (k0 + chunk_even < p.K) ? 0u : kOOB, m_odd = (k0 + chunk_odd < p.K) ? 0u : kOOB;
 #pragma unroll
     for (int i = 0; i < NA; ++i)
-      __builtin_amdgcn_raw_ptr_buffer_load_lds(rsA, (lds_ptr_t)(sA + i * 1024), 16, a_voff[i] | kmask, k0, 0, 0);
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(rsA, (lds_ptr_t)(dst + i * 1024), 16,
+                                               a_voff[i] | (((wave * NA + i) & 1) ? m_odd : m_even), k0, 0, 0);
+  };
+  auto issue_b = [&](int kt) {
+    const int k0 = kt * BK;
+    uint8_t *dst = smem + ((2 * kt + 1) % R) * UNIT + wave * (NB * 1024);
+    const uint32_t m_even = (k0 + chunk_even < p.K) ? 0u : kOOB, m_odd = (k0 + chunk_odd < p.K) ? 0u : kOOB;
 #pragma unroll
     for (int i = 0; i < NB; ++i)
-      __builtin_amdgcn_raw_ptr_buffer_load_lds(rsB, (lds_ptr_t)(sB + i * 1024), 16, b_voff[i] | kmask, k0, 0, 0);
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(rsB, (lds_ptr_t)(dst + i * 1024), 16,
+                                               b_voff[i] | (((wave * NB + i) & 1) ? m_odd : m_even), k0, 0, 0);
+  };
+  auto issue_unit = [&](int u) {
+    if (u & 1) issue_b(u >> 1);
+    else issue_a(u >> 1);
   };
 
   // ---- LDS -> register fragment plan ----
   const int l31 = lane & 31, h = lane >> 5;
-  const int fr = (l31 >> 2) & 3;
-  const int foff0 = l31 * BK + (((h * 2 + 0) ^ fr) * 16);
-  const int foff1 = l31 * BK + (((h * 2 + 1) ^ fr) * 16);
+  const int fr = (l31 & 7) ^ ((l31 >> 3) & 1);
+  int foff[2][2];
+#pragma unroll
+  for (int s = 0; s < 2; ++s)
+#pragma unroll
+    for (int j = 0; j < 2; ++j) foff[s][j] = l31 * BK + (((s * 4 + h * 2 + j) ^ fr) * 16);
   const int a_base = wm * (TM * 32 * BK);
-  const int b_base = A_BYTES + wn * (TN * 32 * BK);
+  const int b_base = wn * (TN * 32 * BK);
 
-  auto read_frags = [&](int kt, v8i (&af)[TM], v8i (&bf)[TN]) {
-    const uint8_t *st = smem + (kt % NS) * STAGE;
+  auto read_frags = [&](int kt, int s, v8i (&af)[TM], v8i (&bf)[TN]) {
+    const uint8_t *pa = smem + ((2 * kt) % R) * UNIT + a_base;
+    const uint8_t *pb = smem + ((2 * kt + 1) % R) * UNIT + b_base;
 #pragma unroll
     for (int tm = 0; tm < TM; ++tm) {
-      const v4i lo = *(const v4i *)(st + a_base + tm * (32 * BK) + foff0);
-      const v4i hi = *(const v4i *)(st + a_base + tm * (32 * BK) + foff1);
+      const v4i lo = *(const v4i *)(pa + tm * (32 * BK) + foff[s][0]);
+      const v4i hi = *(const v4i *)(pa + tm * (32 * BK) + foff[s][1]);
       af[tm] = v8i{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
     }
 #pragma unroll
     for (int tn = 0; tn < TN; ++tn) {
-      const v4i lo = *(const v4i *)(st + b_base + tn * (32 * BK) + foff0);
-      const v4i hi = *(const v4i *)(st + b_base + tn * (32 * BK) + foff1);
+      const v4i lo = *(const v4i *)(pb + tn * (32 * BK) + foff[s][0]);
+      const v4i hi = *(const v4i *)(pb + tn * (32 * BK) + foff[s][1]);
       bf[tn] = v8i{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
     }
   };
@@ -206,60 +233,45 @@ __global__ __launch_bounds__(WM *WN * 64) void gemm_nt_kernel(const GemmArgs p) 
         acc[tn][tm] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(bf[tn], af[tm], acc[tn][tm], 0, 0, 0, 0, 0, 0);
   };
 
-  // Ring bookkeeping.  Tile t lives in stage t % NS; each wave issues LPT
-  // loads per tile, in tile order.  At the top of iteration kt the loads of
-  // tiles kt+1 .. kt+NS-1 may be outstanding; waiting until at most
-  // (NS-2)*LPT remain means this wave's part of tile kt+1 has landed, and the
-  // barrier extends that to every wave.  The same wait also drains this wave's
-  // LDS reads of tile kt (lgkmcnt 0), so after the barrier every wave holds
-  // tile kt in registers and stage kt % NS can be refilled with tile kt+NS.
-  // The empty asm statements keep the compiler from moving LDS accesses across.
-#define L8_PUBLISH_NEXT()                  \
-  do {                                     \
-    L8_WAIT_VM_LGKM0((NS - 2) * LPT);      \
-    asm volatile("" ::: "memory");         \
-    __builtin_amdgcn_s_barrier();          \
-    asm volatile("" ::: "memory");         \
-  } while (0)
-
-  // prologue: all NS stages in flight, tile 0 published and read
+  // prologue: R units in flight, K tile 0 published, its first half read
 #pragma unroll
-  for (int t = 0; t < NS; ++t) issue(t);
+  for (int u = 0; u < R; ++u) issue_unit(u);
   v8i af0[TM], bf0[TN], af1[TM], bf1[TN];
-  L8_WAIT_VM_LGKM0((NS - 1) * LPT);
+  L8_WAIT_VM_LGKM0(PEND0);
   asm volatile("" ::: "memory");
   __builtin_amdgcn_s_barrier();
   asm volatile("" ::: "memory");
-  read_frags(0, af0, bf0);
+  read_frags(0, 0, af0, bf0);
 
-  // Issue order inside one half trip.  A wave issues in order, and right after
-  // the barrier all waves push their LDS reads at once; if those came first,
-  // each wave's matrix-core work would wait behind the whole backlog.  So the
-  // reads (and the global loads) are spread between the MFMAs, which need
-  // nothing but registers that are already valid.
+  // One trip = one K tile of 128 = two matrix-core steps of 64.
+  //   first half : MFMAs on (kt, step 0) while (kt, step 1) is read from LDS;
+  //   barrier    : every wave has now read all of K tile kt (lgkmcnt 0), and
+  //                K tile kt+1 has landed for every wave (partial vmcnt wait),
+  //                so the two slots of K tile kt are refilled with the next
+  //                two units of the sequence;
+  //   second half: MFMAs on (kt, step 1) while (kt+1, step 0) is read.
+  // A wave issues in order, so LDS reads and global loads are spread between
+  // the MFMAs instead of queueing in front of them.
   constexpr int N_MMA = TM * TN, N_DSR = 2 * (TM + TN);
-  auto interleave = [&]() { interleave_step<N_MMA, N_DSR, (L8_GEMM_DIAG == 1 ? 0 : LPT), 0>(); };
-
-  // Two tiles per trip so that the two fragment sets keep fixed registers.  An
-  // odd tile count is rounded up: the extra tile was loaded out of range, i.e.
-  // as zeros, and adds nothing.
-  for (int kt = 0; kt < KT; kt += 2) {
-    // matrix cores on tile kt (set 0) while tile kt+1 is read into set 1
-    L8_PUBLISH_NEXT();
-    if (L8_GEMM_DIAG != 1) issue(kt + NS);
-    if (L8_GEMM_DIAG != 2 && L8_GEMM_DIAG != 4 && L8_GEMM_DIAG != 5) {
-      read_frags(kt + 1, af1, bf1);
+  for (int kt = 0; kt < KT; ++kt) {
+    if (L8_GEMM_DIAG != 2 && L8_GEMM_DIAG != 4) {
+      read_frags(kt, 1, af1, bf1);
       mma(af0, bf0);
-      interleave();
+      interleave_step<N_MMA, N_DSR, 0, 0>();
     }
     __builtin_amdgcn_sched_barrier(0);
-    // matrix cores on tile kt+1 (set 1) while tile kt+2 is read into set 0
-    L8_PUBLISH_NEXT();
-    if (L8_GEMM_DIAG != 1) issue(kt + 1 + NS);
-    if (L8_GEMM_DIAG != 2 && L8_GEMM_DIAG != 4 && L8_GEMM_DIAG != 5) {
-      read_frags(kt + 2, af0, bf0);
+    L8_WAIT_VM_LGKM0(PEND);
+    asm volatile("" ::: "memory");
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
+    if (L8_GEMM_DIAG != 1) {
+      issue_unit(2 * kt + R);
+      issue_unit(2 * kt + R + 1);
+    }
+    if (L8_GEMM_DIAG != 2 && L8_GEMM_DIAG != 4) {
+      read_frags(kt + 1, 0, af0, bf0);
       mma(af1, bf1);
-      interleave();
+      interleave_step<N_MMA, N_DSR, (L8_GEMM_DIAG == 1 ? 0 : NA + NB), 0>();
     }
     __builtin_amdgcn_sched_barrier(0);
   }
@@ -351,25 +363,24 @@ struct Algo {
   int bm, bn, threads, lds;
 };
 
-// X(WM, WN, TM, TN, NS, GROUP_M) -- 1-based position in this list is the `algo` number
-#define L8_ALGO_LIST(X)                                                      \
-  X(2, 4, 4, 2, 4, 8)  /* 1: 256x256, 8 waves (128x64 each), 4 stages     */ \
-  X(2, 4, 4, 2, 5, 8)  /* 2: same, 5 stages (all 160 KiB of LDS)          */ \
-  X(2, 2, 4, 4, 4, 8)  /* 3: 256x256, 4 waves (128x128 each), 4 stages    */ \
-  X(2, 2, 4, 4, 5, 8)  /* 4: same, 5 stages                               */ \
-  X(2, 2, 2, 2, 4, 8)  /* 5: 128x128, 4 waves (small problems)            */ \
-  X(4, 2, 2, 4, 4, 8)  /* 6: 256x256, 8 waves (64x128 each), 4 stages     */ \
-  X(2, 4, 4, 2, 3, 8)  /* 7: algo 1 with 3 stages                         */ \
-  X(2, 4, 4, 2, 4, 4)  /* 8: algo 1 with shorter groups                   */ \
-  X(2, 4, 4, 2, 4, 16) /* 9: algo 1 with taller groups                    */
+// X(WM, WN, TM, TN, R, GROUP_M) -- 1-based position in this list is the `algo` number
+#define L8_ALGO_LIST(X)                                                       \
+  X(2, 4, 4, 2, 5, 4)  /* 1: 256x256, 8 waves (128x64 each), ring of 5     */ \
+  X(2, 4, 4, 2, 4, 4)  /* 2: same, ring of 4 (two whole K tiles)           */ \
+  X(2, 2, 4, 4, 5, 4)  /* 3: 256x256, 4 waves (128x128 each), ring of 5    */ \
+  X(4, 2, 2, 4, 5, 4)  /* 4: 256x256, 8 waves (64x128 each), ring of 5     */ \
+  X(2, 2, 2, 2, 5, 4)  /* 5: 128x128, 4 waves (small problems)             */ \
+  X(2, 4, 4, 2, 5, 8)  /* 6: algo 1 with taller groups                     */ \
+  X(2, 4, 4, 2, 5, 2)  /* 7: algo 1 with shorter groups                    */
 
-#define L8_INSTANTIATE(WM, WN, TM, TN, NS, GM) \
-  template __global__ void gemm_nt_kernel<WM, WN, TM, TN, NS, GM>(const GemmArgs);
+#define L8_INSTANTIATE(WM, WN, TM, TN, R, GM) \
+  template __global__ void gemm_nt_kernel<WM, WN, TM, TN, R, GM>(const GemmArgs);
 L8_ALGO_LIST(L8_INSTANTIATE)
 
-#define L8_ALGO_ROW(WM, WN, TM, TN, NS, GM)                                                        \
-  {"mt" #WM "x" #WN "w_" #TM "x" #TN "t_ns" #NS "_g" #GM, gemm_nt_kernel<WM, WN, TM, TN, NS, GM>, \
-   WM * TM * 32, WN * TN * 32, WM * WN * 64, NS * (WM * TM * 32 + WN * TN * 32) * 64},
+#define L8_MAX2(a, b) ((a) > (b) ? (a) : (b))
+#define L8_ALGO_ROW(WM, WN, TM, TN, R, GM)                                                      \
+  {"mt" #WM "x" #WN "w_" #TM "x" #TN "t_r" #R "_g" #GM, gemm_nt_kernel<WM, WN, TM, TN, R, GM>, \
+   WM * TM * 32, WN * TN * 32, WM * WN * 64, R * L8_MAX2(WM * TM * 32, WN * TN * 32) * 128},
 
 static const Algo kAlgos[] = {L8_ALGO_LIST(L8_ALGO_ROW)};
 constexpr int kNumAlgos = sizeof(kAlgos) / sizeof(kAlgos[0]);
