@@ -26,6 +26,9 @@ DIM, FFN, TOKENS = 4096, 11008, 16384
 STEP_FLOP = 18 * TOKENS * DIM * FFN          # 9 GEMMs x 2*M*N*K
 PEAK_FP8_TFLOPS = 5000.0                     # MI355X dense fp8 MFMA, published
 PEAK_HBM_GBPS = 8000.0                       # MI355X HBM3E, published
+# HBM-side bytes per forward-shape GEMM launch from rocprofv3 FETCH_SIZE / WRITE_SIZE, each scaled by what the
+# same counter reads for a 256 MiB copy (profiles/gemm_nt_7b_fwd_hbm_traffic.txt): 1.126 GB read + 0.440 GB written
+GEMM_TRAFFIC_BYTES = 1_566_000_000
 
 
 def parse():
@@ -37,6 +40,9 @@ def parse():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-sample-tokens", type=int, default=2048)
     ap.add_argument("--no-kernel-timing", action="store_true", help="do not record per-kernel events in the timed steps")
+    ap.add_argument("--kernel-only", choices=["gemm", "copy"], default=None,
+                    help="profiling aid: launch only the forward-shape GEMM, or a plain 256 MiB device copy "
+                         "(the reference point the FETCH_SIZE / WRITE_SIZE counters are scaled by), a few times")
     return ap.parse_args()
 
 
@@ -108,6 +114,29 @@ def main():
     torch.cuda.set_device(dev)
     f8.config.gemm_algo = args.algo
 
+    if args.kernel_only == "copy":
+        n = 256 << 20
+        src = torch.ones(n, dtype=torch.uint8, device=dev)
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        print(json.dumps({"kernel_only": "copy", "bytes_read": n, "bytes_written": n, "launches": 3}))
+        return
+    if args.kernel_only == "gemm":
+        g = torch.Generator().manual_seed(2)
+        a = torch.randn(TOKENS, DIM, generator=g).to(torch.bfloat16).to(dev)
+        b = (torch.randn(FFN, DIM, generator=g) * 0.02).to(torch.bfloat16).to(dev)
+        qa, sa, _ = ops.cast_rowwise(a)
+        qb, sb, _ = ops.cast_rowwise(b)
+        out = torch.empty(TOKENS, FFN, dtype=torch.bfloat16, device=dev)
+        for _ in range(3):
+            ops.gemm_nt(qa, qb, sa, sb, algo=args.algo, out=out)
+        torch.cuda.synchronize()
+        print(json.dumps({"kernel_only": "gemm", "M": TOKENS, "N": FFN, "K": DIM, "launches": 3,
+                          "algorithmic_bytes": TOKENS * DIM + FFN * DIM + 2 * TOKENS * FFN + 4 * (TOKENS + FFN)}))
+        return
+
     mlp = make_mlp(torch, nn, DIM, FFN, dev)
     model = convert_linears_to_fp8(nn.ModuleDict({"layers": nn.ModuleList([mlp])}), "rowwise", r"layers\.[0-9]+\.")
     mlp = model["layers"][0]
@@ -160,7 +189,8 @@ def main():
         achieved = work / (ms * 1e-3) / 1e12
         roofline = {"kernel": "gemm_nt_kernel (fp8 e4m3 NT GEMM, 2*16384*4096*11008 flop per launch)",
                     "bound": "mfma", "achieved": round(achieved, 1), "peak": PEAK_FP8_TFLOPS, "unit": "TFLOP/s",
-                    "frac": round(achieved / PEAK_FP8_TFLOPS, 4), "traffic": None}
+                    "frac": round(achieved / PEAK_FP8_TFLOPS, 4), "traffic": GEMM_TRAFFIC_BYTES,
+                    "traffic_unit": "bytes per launch (algorithmic: 473 MB)"}
 
     out = {
         "metric": "fp8 rowwise linear fwd+bwd TFLOP/s at 7B MLP",
