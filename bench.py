@@ -40,6 +40,9 @@ def parse():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-sample-tokens", type=int, default=2048)
     ap.add_argument("--no-kernel-timing", action="store_true", help="do not record per-kernel events in the timed steps")
+    ap.add_argument("--workload", choices=["mlp7b", "llama1b"], default="mlp7b",
+                    help="mlp7b = the headline workload; llama1b = full Llama-1B-shaped forward+backward step "
+                         "(25 layers, dim 2048, ffn 8192, vocab 128256, 4 x 4096 tokens), reported in tokens/s")
     ap.add_argument("--kernel-only", choices=["gemm", "copy"], default=None,
                     help="profiling aid: launch only the forward-shape GEMM, or a plain 256 MiB device copy "
                          "(the reference point the FETCH_SIZE / WRITE_SIZE counters are scaled by), a few times")
@@ -96,6 +99,44 @@ def cpu_baseline(torch, sample_tokens):
     }
 
 
+def run_llama1b(args, torch, dev):
+    """configs[4]: tokens/s of a Llama-1B-shaped forward+backward step, block linears in row-wise fp8."""
+    from lingua_amd import convert_linears_to_fp8
+    from lingua_amd.callers import Llama, LLAMA_1B, llama_flops_per_token
+    B, S = 4, 4096
+    with torch.device(dev):
+        model = Llama(**LLAMA_1B).to(torch.bfloat16)
+    model.init_weights(0.02, seed=0)
+    model = convert_linears_to_fp8(model, "rowwise", r"layers\.[0-9]+\.")
+    g = torch.Generator().manual_seed(0)
+    tokens = torch.randint(0, LLAMA_1B["vocab"], (B, S), generator=g).to(dev)
+    labels = torch.randint(0, LLAMA_1B["vocab"], (B, S), generator=g).to(dev)
+
+    def step():
+        for p in model.parameters():
+            p.grad = None
+        model(tokens, labels).backward()
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    dt = (time.perf_counter() - t0) / args.steps
+    fpt = llama_flops_per_token(LLAMA_1B["n_layers"], LLAMA_1B["dim"], LLAMA_1B["ffn_dim"], LLAMA_1B["vocab"], S)
+    fp8_flop = 25 * 3 * (4 * 2 * B * S * 2048 * 2048 + 3 * 2 * B * S * 2048 * 8192)
+    print(json.dumps({
+        "metric": "Llama-1B forward+backward tokens/s, block linears fp8 row-wise", "value": round(B * S / dt, 1),
+        "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(dt * 1e3, 3),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "fp8_e4m3fn", "data": "synthetic",
+        "config": {"workload": "llama-1B step fwd+bwd (configs[4])", "batch": B, "seq_len": S, **LLAMA_1B},
+        "model_TFLOP/s": round(fpt * B * S / dt / 1e12, 1),
+        "fp8_linear_TFLOP/s_if_alone": round(fp8_flop / dt / 1e12, 1),
+    }))
+
+
 def main():
     args = parse()
     if args.gpus != 1:
@@ -135,6 +176,10 @@ def main():
         torch.cuda.synchronize()
         print(json.dumps({"kernel_only": "gemm", "M": TOKENS, "N": FFN, "K": DIM, "launches": 3,
                           "algorithmic_bytes": TOKENS * DIM + FFN * DIM + 2 * TOKENS * FFN + 4 * (TOKENS + FFN)}))
+        return
+
+    if args.workload == "llama1b":
+        run_llama1b(args, torch, dev)
         return
 
     mlp = make_mlp(torch, nn, DIM, FFN, dev)

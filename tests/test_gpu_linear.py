@@ -197,3 +197,54 @@ def test_outlier_stress_rowwise_beats_tensorwise_on_the_linear():
     e_ten = rel_l2(y_ten, exact)
     assert e_row < e_ten
     assert (y_row[zr.cuda()] == 0).all()                      # all-zero token rows give exact zeros
+
+
+def test_config5_llama_1b_training_step():
+    # full Llama-1B-shaped step (25 layers, dim 2048, 16 heads, ffn 8192, vocab 128256, 4 x 4096 tokens), all block
+    # linears fp8 row-wise, output head bf16; three linears are checked against the oracle through hooks
+    from lingua_amd import convert_linears_to_fp8, Fp8Linear
+    from lingua_amd.callers import Llama, LLAMA_1B
+    torch.manual_seed(0)
+    with torch.device("cuda"):
+        model = Llama(**LLAMA_1B).to(torch.bfloat16)
+    model.init_weights(0.02, seed=0)
+    g = torch.Generator().manual_seed(0)
+    tokens = torch.randint(0, LLAMA_1B["vocab"], (4, 4096), generator=g).cuda()
+    labels = torch.randint(0, LLAMA_1B["vocab"], (4, 4096), generator=g).cuda()
+    with torch.no_grad():
+        loss_bf16 = float(model(tokens, labels))
+    keys_before = list(model.state_dict().keys())
+    model = convert_linears_to_fp8(model, "rowwise", r"layers\.[0-9]+\.")
+    n_fp8 = sum(1 for m in model.modules() if type(m) is Fp8Linear)
+    assert n_fp8 == 25 * 7
+    assert type(model.output) is nn.Linear and list(model.state_dict().keys()) == keys_before
+
+    picks = {"layers.0.attention.wq": None, "layers.12.feed_forward.w2": None, "layers.24.feed_forward.w1": None}
+    seen, hooks = {}, []
+    mods = dict(model.named_modules())
+    for name in picks:
+        m = mods[name]
+        hooks.append(m.register_forward_hook(
+            lambda m_, inp, out, name=name: seen.__setitem__(name + ":io", (inp[0].detach(), out.detach()))))
+        hooks.append(m.register_full_backward_hook(
+            lambda m_, gin, gout, name=name: seen.__setitem__(name + ":g", (gin[0].detach(), gout[0].detach()))))
+    loss = model(tokens, labels)
+    loss.backward()
+    for h_ in hooks:
+        h_.remove()
+    assert torch.isfinite(loss) and abs(float(loss) - loss_bf16) < 0.05 * abs(loss_bf16)
+    rows = torch.arange(0, 16384, 16384 // 16)[:16].cuda()
+    for name in picks:
+        lin = mods[name]
+        W = lin.weight.detach().cpu()
+        a_in, out = (t.flatten(0, 1) for t in seen[name + ":io"])
+        g_in, g_out = (t.flatten(0, 1) for t in seen[name + ":g"])
+        assert rel_l2(out[rows], oracle.linear_forward(a_in[rows].cpu(), W)) <= TOL, name
+        assert rel_l2(g_in[rows], oracle.linear_dgrad(g_out[rows].cpu(), W)) <= TOL, name
+        n_idx = torch.arange(0, W.shape[0], max(1, W.shape[0] // 24))[:24].cuda()
+        k_idx = torch.arange(0, W.shape[1], max(1, W.shape[1] // 24))[:24].cuda()
+        qg, sg = oracle.cast_colwise_transposed(g_out[:, n_idx].cpu())
+        qa, sa = oracle.cast_colwise_transposed(a_in[:, k_idx].cpu())
+        want = oracle.gemm_nt(qg, qa, sg, sa)
+        assert rel_l2(lin.weight.grad[n_idx][:, k_idx], want) <= TOL, name
+    assert all(p.grad is not None and torch.isfinite(p.grad.float()).all() for p in model.parameters())
