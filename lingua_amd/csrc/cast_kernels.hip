@@ -30,10 +30,13 @@ L8_DEV void load_row(v4i (&buf)[NCH], const uint16_t *row, int C, int lane) {
 }
 
 template <int NCH, bool COLMAX>
-__global__ __launch_bounds__(kRowBlock) void cast_rowwise_kernel(
+__global__ __launch_bounds__(kRowBlock, 2) void cast_rowwise_kernel(
     const uint16_t *__restrict__ x, int64_t R, int C, int64_t ldx, uint8_t *__restrict__ q, int64_t ldq,
     float *__restrict__ scale, uint16_t *__restrict__ amax_out, uint32_t *__restrict__ col_amax) {
-  extern __shared__ uint32_t lds_colmax[];  // [C] when COLMAX
+  extern __shared__ uint32_t lds_colmax[];  // [C/2] packed bf16 pairs when COLMAX
+  // the next row is prefetched into a second register set unless that would
+  // push the wave beyond 256 VGPRs (two waves per SIMD are worth more)
+  constexpr bool PREFETCH = COLMAX ? (NCH <= 8) : (NCH <= 24);
   const int lane = threadIdx.x & 63;
   const int wave = threadIdx.x >> 6;
   const int64_t wave_stride = (int64_t)gridDim.x * kRowWaves;
@@ -43,15 +46,14 @@ __global__ __launch_bounds__(kRowBlock) void cast_rowwise_kernel(
   if (COLMAX) {
 #pragma unroll
     for (int i = 0; i < NCH * 4; ++i) cmax[i] = 0;
-    for (int c = threadIdx.x; c < C; c += kRowBlock) lds_colmax[c] = 0;
   }
 
   v4i cur[NCH];
   if (r < R) load_row<NCH>(cur, x + r * ldx, C, lane);
   while (r < R) {
     const int64_t rn = r + wave_stride;
-    v4i nxt[NCH];
-    if (rn < R) load_row<NCH>(nxt, x + rn * ldx, C, lane);
+    v4i nxt[PREFETCH ? NCH : 1];
+    if (PREFETCH && rn < R) load_row<PREFETCH ? NCH : 1>(nxt, x + rn * ldx, C, lane);
 
     // row amax on packed pairs
     uint32_t m = 0;
@@ -94,29 +96,141 @@ __global__ __launch_bounds__(kRowBlock) void cast_rowwise_kernel(
         }
       }
     }
+    if (PREFETCH) {
 #pragma unroll
-    for (int j = 0; j < NCH; ++j) cur[j] = nxt[j];
+      for (int j = 0; j < NCH; ++j) cur[j] = nxt[PREFETCH ? j : 0];
+    } else if (rn < R) {
+      __builtin_amdgcn_sched_barrier(0);  // the row registers are reused: do not start the loads early
+      load_row<NCH>(cur, x + rn * ldx, C, lane);
+    }
     r = rn;
   }
 
   if (COLMAX) {
-    __syncthreads();  // lds_colmax zero-filled
+    // merge the four waves' column maxima through LDS, one wave after the other
+    // (packed pairs, plain reads and writes), then raise the global values:
+    // a plain read first, the atomic only where this workgroup has a larger
+    // value -- late workgroups rarely do, so atomics stay rare.  A stale read
+    // can only cause a redundant atomic, never a missed one.
+    v4i *lds4 = (v4i *)lds_colmax;
+    for (int w = 0; w < kRowWaves; ++w) {
+      if (wave == w) {
 #pragma unroll
-    for (int j = 0; j < NCH; ++j) {
-      const int c = j * 512 + lane * 8;
-      if (c < C) {
+        for (int j = 0; j < NCH; ++j) {
+          const int c = j * 512 + lane * 8;
+          if (c < C) {
+            v4i mine = {(int)cmax[j * 4], (int)cmax[j * 4 + 1], (int)cmax[j * 4 + 2], (int)cmax[j * 4 + 3]};
+            if (w > 0) {
+              const v4i old = lds4[c / 8];
 #pragma unroll
-        for (int k = 0; k < 4; ++k) {
-          const uint32_t v = cmax[j * 4 + k];
-          atomicMax(&lds_colmax[c + 2 * k], (v & 0xffffu) << 16);       // bf16 -> fp32 bit pattern
-          atomicMax(&lds_colmax[c + 2 * k + 1], v & 0xffff0000u);
+              for (int k = 0; k < 4; ++k) mine[k] = (int)pk_absmax_u16((uint32_t)old[k], (uint32_t)mine[k]);
+            }
+            lds4[c / 8] = mine;
+          }
+        }
+      }
+      __syncthreads();
+    }
+    for (int i = threadIdx.x; i < C / 2; i += kRowBlock) {
+      const uint32_t v = lds_colmax[i];
+      const uint32_t lo = (v & 0xffffu) << 16, hi = v & 0xffff0000u;  // bf16 -> fp32 bit patterns
+      const uint32_t g0 = __builtin_nontemporal_load(&col_amax[2 * i]);
+      const uint32_t g1 = __builtin_nontemporal_load(&col_amax[2 * i + 1]);
+      if (lo > g0) atomicMax(&col_amax[2 * i], lo);
+      if (hi > g1) atomicMax(&col_amax[2 * i + 1], hi);
+    }
+  }
+}
+
+// Long rows: the four waves of a workgroup share one row (wave w owns chunks
+// w, w+4, w+8, ... of 512 columns), so a lane holds at most NCHW chunks and
+// many workgroups fit a CU.  The row amax crosses waves through LDS with one
+// barrier per row (double-buffered).  Column maxima of different waves cover
+// disjoint columns and are merged into the global array directly.
+template <int NCHW, bool COLMAX>
+__global__ __launch_bounds__(kRowBlock, (NCHW <= 4 ? 4 : (NCHW <= 8 ? 2 : 1))) void cast_rowwise_wg_kernel(
+    const uint16_t *__restrict__ x, int64_t R, int C, int64_t ldx, uint8_t *__restrict__ q, int64_t ldq,
+    float *__restrict__ scale, uint16_t *__restrict__ amax_out, uint32_t *__restrict__ col_amax) {
+  __shared__ uint32_t red[2][kRowWaves];
+  const int lane = threadIdx.x & 63;
+  const int wave = threadIdx.x >> 6;
+  auto col_of = [&](int j) { return (j * kRowWaves + wave) * 512 + lane * 8; };
+  auto load = [&](v4i (&buf)[NCHW], int64_t r) {
+#pragma unroll
+    for (int j = 0; j < NCHW; ++j) {
+      const int c = col_of(j);
+      if (c < C) buf[j] = __builtin_nontemporal_load((const v4i *)(x + r * ldx + c));
+      else buf[j] = v4i{0, 0, 0, 0};
+    }
+  };
+  uint32_t cmax[COLMAX ? NCHW * 4 : 1];
+  if (COLMAX) {
+#pragma unroll
+    for (int i = 0; i < NCHW * 4; ++i) cmax[i] = 0;
+  }
+  int64_t r = blockIdx.x;
+  v4i cur[NCHW], nxt[NCHW];
+  if (r < R) load(cur, r);
+  for (int it = 0; r < R; ++it) {
+    const int64_t rn = r + gridDim.x;
+    if (rn < R) load(nxt, rn);
+    uint32_t m = 0;
+#pragma unroll
+    for (int j = 0; j < NCHW; ++j)
+#pragma unroll
+      for (int k = 0; k < 4; ++k) {
+        m = pk_absmax_u16(m, (uint32_t)cur[j][k]);
+        if (COLMAX) cmax[j * 4 + k] = pk_absmax_u16(cmax[j * 4 + k], (uint32_t)cur[j][k]);
+      }
+    m = wave_max_u32(max(m & 0xffffu, m >> 16));
+    if (lane == 0) red[it & 1][wave] = m;
+    __syncthreads();
+    uint32_t amax_bits = 0;
+#pragma unroll
+    for (int w = 0; w < kRowWaves; ++w) amax_bits = max(amax_bits, red[it & 1][w]);
+    const bool finite = amax_bits < 0x7f80u;
+    float s;
+    if (finite) s = scale_from_amax(bf16_bits_to_f32(amax_bits));
+    else s = __uint_as_float(amax_bits == 0x7f80u ? 0x7f800000u : 0x7fc00000u);
+    const float recip = recip_exact(s);
+    if (threadIdx.x == 0) {
+      if (scale) scale[r] = s;
+      if (amax_out) amax_out[r] = (uint16_t)amax_bits;
+    }
+    if (q) {
+      uint8_t *qrow = q + r * ldq;
+#pragma unroll
+      for (int j = 0; j < NCHW; ++j) {
+        const int c = col_of(j);
+        if (c < C) {
+          if (finite) __builtin_nontemporal_store(cvt8(cur[j], recip), (v2i *)(qrow + c));
+          else *(v2i *)(qrow + c) = cvt8_slow(cur[j], recip);
         }
       }
     }
-    __syncthreads();
-    for (int c = threadIdx.x; c < C; c += kRowBlock) {
-      const uint32_t v = lds_colmax[c];
-      if (v) atomicMax(&col_amax[c], v);
+#pragma unroll
+    for (int j = 0; j < NCHW; ++j) cur[j] = nxt[j];
+    r = rn;
+  }
+  if (COLMAX) {
+    // plain read first, atomic only where this workgroup has a larger value (a
+    // stale read can only cause a redundant atomic, never a missed one)
+#pragma unroll
+    for (int j = 0; j < NCHW; ++j) {
+      const int c = col_of(j);
+      if (c < C) {
+        const v4i g0 = __builtin_nontemporal_load((const v4i *)(col_amax + c));
+        const v4i g1 = __builtin_nontemporal_load((const v4i *)(col_amax + c + 4));
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+          const uint32_t v = cmax[j * 4 + k];
+          const uint32_t lo = (v & 0xffffu) << 16, hi = v & 0xffff0000u;
+          const uint32_t glo = (uint32_t)(k < 2 ? g0[2 * k] : g1[2 * k - 4]);
+          const uint32_t ghi = (uint32_t)(k < 2 ? g0[2 * k + 1] : g1[2 * k - 3]);
+          if (lo > glo) atomicMax(&col_amax[c + 2 * k], lo);
+          if (hi > ghi) atomicMax(&col_amax[c + 2 * k + 1], hi);
+        }
+      }
     }
   }
 }
@@ -192,16 +306,19 @@ __global__ __launch_bounds__(256) void col_amax_kernel(const uint16_t *__restric
   }
 }
 
-// bf16 amax[n] -> bf16 amax_out[1]; one workgroup.
-__global__ __launch_bounds__(256) void amax_reduce_kernel(const uint16_t *__restrict__ amax, int64_t n,
-                                                          uint16_t *__restrict__ out) {
-  __shared__ uint32_t red[4];
+// bf16 amax[n] -> bf16 amax_out[1]; one workgroup of 1024 threads.
+__global__ __launch_bounds__(1024) void amax_reduce_kernel(const uint16_t *__restrict__ amax, int64_t n,
+                                                           uint16_t *__restrict__ out) {
+  __shared__ uint32_t red[16];
   uint32_t m = 0;
-  for (int64_t i = threadIdx.x; i < n; i += 256) m = max(m, (uint32_t)(amax[i] & 0x7fffu));
+  for (int64_t i = threadIdx.x; i < n; i += 1024) m = max(m, (uint32_t)(amax[i] & 0x7fffu));
   m = wave_max_u32(m);
   if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = m;
   __syncthreads();
-  if (threadIdx.x == 0) out[0] = (uint16_t)max(max(red[0], red[1]), max(red[2], red[3]));
+  if (threadIdx.x < 64) {
+    m = wave_max_u32(threadIdx.x < 16 ? red[threadIdx.x] : 0u);
+    if (threadIdx.x == 0) out[0] = (uint16_t)m;
+  }
 }
 
 // ---------------------------------------------------------------------------
@@ -239,13 +356,24 @@ __global__ __launch_bounds__(256) void cast_tensorwise_kernel(const uint16_t *__
 
 // ---------------------------------------------------------------------------
 // Transposed casts (tensor-wise for the dgrad weight, column-wise for wgrad):
-// a [128 rows x 64 cols] tile of x becomes a [64 x 128] tile of q.
+// a [256 rows x 64 cols] tile of x becomes a [64 x 256] tile of q.
 // Thread t loads 8 columns (one 16-byte load) from each of 4 consecutive rows,
 // packs, for each of its 8 columns, the 4 row-consecutive e4m3 bytes into one
 // dword and writes it to the transposed tile in LDS; the tile is then read
-// back as 16-byte row segments and stored with full 128-byte output rows.
+// back as 16-byte row segments and stored as 256-byte runs of the output rows.
 // ---------------------------------------------------------------------------
-constexpr int kTR = 128, kTC = 64, kTStride = kTR + 16;  // LDS row stride in bytes
+#ifndef L8_TC
+#define L8_TC 64
+#endif
+#ifndef L8_TU
+#define L8_TU 2
+#endif
+constexpr int kTC = L8_TC;                   // columns of x per tile
+constexpr int kCCH = kTC / 8;                // 8-column chunks per tile row
+constexpr int kRG = 256 / kCCH;              // 4-row groups covered by the 256 threads in one pass
+constexpr int kTU = L8_TU;                   // passes (4-row units per thread)
+constexpr int kTR = kRG * 4 * kTU;           // rows of x per tile
+constexpr int kTStride = kTR + 16;           // LDS row stride in bytes
 
 template <bool PER_COL>
 __global__ __launch_bounds__(256) void cast_transposed_kernel(
@@ -255,28 +383,51 @@ __global__ __launch_bounds__(256) void cast_transposed_kernel(
   __shared__ __attribute__((aligned(16))) uint8_t tile[kTC * kTStride];
   __shared__ float recips[kTC];
   const int t = threadIdx.x;
-  const int64_t r0 = (int64_t)blockIdx.y * kTR;
-  const int c0 = blockIdx.x * kTC;
+  // Workgroup w takes column block w % nct and row tile (w / nct + w % nct) % nrt:
+  // a diagonal walk.  The workgroups resident at one time then touch addresses
+  // that differ in their low bits on both sides, which keeps power-of-two row
+  // strides (input stride C, output stride R) from piling onto a few memory
+  // channels, while each column block still advances through consecutive row
+  // tiles (long runs in the output rows) and each row tile through consecutive
+  // column blocks (wide bands of the input rows).
+  const int nct = (C + kTC - 1) / kTC;
+  const int64_t nrt = (R + kTR - 1) / kTR;
+  const int cb = (int)(blockIdx.x % nct);
+  const int64_t rt = (blockIdx.x / nct + cb) % nrt;
+  const int64_t r0 = rt * kTR;
+  const int c0 = cb * kTC;
+  const int cc = t % kCCH;  // which 8-column chunk of the tile
+  const int rg = t / kCCH;  // which 4-row group of a pass
+  const int c = c0 + cc * 8;
+
+  // issue the loads first: kTU units of 4 rows x 8 columns per thread
+  v4i in[kTU][4];
+#pragma unroll
+  for (int u = 0; u < kTU; ++u)
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int64_t r = r0 + (u * kRG + rg) * 4 + i;
+      if (r < R && c < C) in[u][i] = __builtin_nontemporal_load((const v4i *)(x + r * ldx + c));
+      else in[u][i] = v4i{0, 0, 0, 0};
+    }
 
   bool finite = true;
   if (PER_COL) {
     if (t < kTC) {
-      const int c = c0 + t;
+      const int col = c0 + t;
       float rc = 0.0f;
-      if (c < C) {
-        const uint32_t bits = col_amax[c];
+      if (col < C) {
+        const uint32_t bits = col_amax[col];
         const float s = scale_from_amax_bits32(bits);
         rc = recip_exact(s);
         if (bits >= 0x7f800000u) rc = __uint_as_float(0x7fc00000u);  // flag: slow path for this column
-        if (blockIdx.y == 0) scale[c] = s;
+        if (rt == 0) scale[col] = s;
       }
       recips[t] = rc;
     }
     __syncthreads();
   }
   float rcp[8];
-  const int cc = t & 7;    // which 8-column chunk of the tile
-  const int rg = t >> 3;   // which 4-row group of the tile (0..31)
   if (PER_COL) {
 #pragma unroll
     for (int j = 0; j < 8; ++j) rcp[j] = recips[cc * 8 + j];
@@ -287,57 +438,52 @@ __global__ __launch_bounds__(256) void cast_transposed_kernel(
     const float rc = recip_exact(s);
 #pragma unroll
     for (int j = 0; j < 8; ++j) rcp[j] = rc;
-    if (blockIdx.x == 0 && blockIdx.y == 0 && t == 0) scale[0] = s;
+    if (blockIdx.x == 0 && t == 0) scale[0] = s;
   }
 
-  // load 4 rows x 8 cols
-  v4i in[4];
-  const int c = c0 + cc * 8;
+  // convert and transpose inside the thread: column j <- rows 0..3 of each unit
 #pragma unroll
-  for (int i = 0; i < 4; ++i) {
-    const int64_t r = r0 + rg * 4 + i;
-    if (r < R && c < C) in[i] = __builtin_nontemporal_load((const v4i *)(x + r * ldx + c));
-    else in[i] = v4i{0, 0, 0, 0};
-  }
-  // convert and transpose inside the thread: column j <- rows 0..3
+  for (int u = 0; u < kTU; ++u)
 #pragma unroll
-  for (int j = 0; j < 8; ++j) {
-    const int w = j >> 1;
-    const bool hi = j & 1;
-    float v[4];
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const uint32_t p = (uint32_t)in[i][w];
-      v[i] = __uint_as_float(hi ? (p & 0xffff0000u) : (p << 16)) * rcp[j];
-    }
-    int packed;
-    const bool fast = PER_COL ? (rcp[j] == rcp[j]) : finite;
-    if (fast) {
-      packed = __builtin_amdgcn_cvt_pk_fp8_f32(v[0], v[1], 0, false);
-      packed = __builtin_amdgcn_cvt_pk_fp8_f32(v[2], v[3], packed, true);
-    } else {
-      // non-finite amax: redo the products with the true reciprocal (0 for inf, NaN for NaN)
-      float rc = rcp[j];
-      if (PER_COL) {
-        const uint32_t bits = col_amax[c + j < C ? c + j : 0];
-        rc = recip_exact(scale_from_amax_bits32(bits));
-      }
-      packed = 0;
+    for (int j = 0; j < 8; ++j) {
+      const int w = j >> 1;
+      const bool hi = j & 1;
+      float v[4];
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
-        const uint32_t p = (uint32_t)in[i][w];
-        const float val = __uint_as_float(hi ? (p & 0xffff0000u) : (p << 16)) * rc;
-        packed |= (int)(e4m3fn_from_f32_slow(val) << (8 * i));
+        const uint32_t p = (uint32_t)in[u][i][w];
+        v[i] = __uint_as_float(hi ? (p & 0xffff0000u) : (p << 16)) * rcp[j];
       }
-    }
-    *(int *)(tile + (cc * 8 + j) * kTStride + rg * 4) = packed;
-  }
-  __syncthreads();
-  // write out: 64 output rows (columns of x) x 128 bytes
+      int packed;
+      const bool fast = PER_COL ? (rcp[j] == rcp[j]) : finite;
+      if (fast) {
+        packed = __builtin_amdgcn_cvt_pk_fp8_f32(v[0], v[1], 0, false);
+        packed = __builtin_amdgcn_cvt_pk_fp8_f32(v[2], v[3], packed, true);
+      } else {
+        // non-finite amax: redo the products with the true reciprocal (0 for inf, NaN for NaN)
+        float rc = rcp[j];
+        if (PER_COL) {
+          const uint32_t bits = col_amax[c + j < C ? c + j : 0];
+          rc = recip_exact(scale_from_amax_bits32(bits));
+        }
+        packed = 0;
 #pragma unroll
-  for (int i = 0; i < 2; ++i) {
-    const int oc = (t >> 3) + i * 32;  // output row within the tile
-    const int seg = t & 7;             // 16-byte segment
+        for (int i = 0; i < 4; ++i) {
+          const uint32_t p = (uint32_t)in[u][i][w];
+          const float val = __uint_as_float(hi ? (p & 0xffff0000u) : (p << 16)) * rc;
+          packed |= (int)(e4m3fn_from_f32_slow(val) << (8 * i));
+        }
+      }
+      *(int *)(tile + (cc * 8 + j) * kTStride + (u * kRG + rg) * 4) = packed;
+    }
+  __syncthreads();
+  // write out: 64 output rows (columns of x) x kTR bytes, 16 bytes per thread and step
+  constexpr int SEGS = kTR / 16;  // 16-byte segments per output row
+#pragma unroll
+  for (int i = 0; i < kTC * SEGS / 256; ++i) {
+    const int idx = i * 256 + t;
+    const int oc = idx / SEGS;   // output row within the tile
+    const int seg = idx % SEGS;
     const int col = c0 + oc;
     const int64_t r = r0 + seg * 16;
     if (col < C && r < R) {
@@ -362,10 +508,10 @@ static int launch_rowwise(const void *x, int64_t R, int64_t C, int64_t ldx, void
   const int cus = num_cus();
   int64_t blocks = (R + kRowWaves - 1) / kRowWaves;
   // with the column-amax by-product fewer, longer-lived workgroups mean fewer merges
-  const int64_t cap = (int64_t)cus * (col_amax ? 4 : 8);
+  const int64_t cap = (int64_t)cus * (col_amax ? 2 : 8);
   if (blocks > cap) blocks = cap;
   if (col_amax) {
-    const size_t lds = (size_t)C * sizeof(uint32_t);
+    const size_t lds = (size_t)C * sizeof(uint16_t);
     hipLaunchKernelGGL((cast_rowwise_kernel<NCH, true>), dim3((unsigned)blocks), dim3(kRowBlock), lds, st,
                        (const uint16_t *)x, R, (int)C, ldx, (uint8_t *)q, ldq, scale, (uint16_t *)amax,
                        (uint32_t *)col_amax);
@@ -374,6 +520,24 @@ static int launch_rowwise(const void *x, int64_t R, int64_t C, int64_t ldx, void
                        (const uint16_t *)x, R, (int)C, ldx, (uint8_t *)q, ldq, scale, (uint16_t *)amax,
                        (uint32_t *)nullptr);
   }
+  L8_HIP(hipGetLastError());
+  return L8_OK;
+}
+
+template <int NCHW>
+static int launch_rowwise_wg(const void *x, int64_t R, int64_t C, int64_t ldx, void *q, int64_t ldq, float *scale,
+                             void *amax, float *col_amax, hipStream_t st) {
+  int64_t blocks = R;
+  const int64_t cap = (int64_t)num_cus() * (col_amax ? 4 : 8);
+  if (blocks > cap) blocks = cap;
+  if (col_amax)
+    hipLaunchKernelGGL((cast_rowwise_wg_kernel<NCHW, true>), dim3((unsigned)blocks), dim3(kRowBlock), 0, st,
+                       (const uint16_t *)x, R, (int)C, ldx, (uint8_t *)q, ldq, scale, (uint16_t *)amax,
+                       (uint32_t *)col_amax);
+  else
+    hipLaunchKernelGGL((cast_rowwise_wg_kernel<NCHW, false>), dim3((unsigned)blocks), dim3(kRowBlock), 0, st,
+                       (const uint16_t *)x, R, (int)C, ldx, (uint8_t *)q, ldq, scale, (uint16_t *)amax,
+                       (uint32_t *)nullptr);
   L8_HIP(hipGetLastError());
   return L8_OK;
 }
@@ -399,8 +563,13 @@ extern "C" int l8_cast_rowwise(const void *x, int64_t R, int64_t C, int64_t ldx,
   const int64_t nch = (C + 511) / 512;
   if (nch <= 4) return launch_rowwise<4>(x, R, C, ldx, q, ldq, scale, amax, col_amax, st);
   if (nch <= 8) return launch_rowwise<8>(x, R, C, ldx, q, ldq, scale, amax, col_amax, st);
-  if (nch <= 16 && !(col_amax && C > 16000)) return launch_rowwise<16>(x, R, C, ldx, q, ldq, scale, amax, col_amax, st);
-  if (nch <= 24 && !(col_amax && C > 16000)) return launch_rowwise<24>(x, R, C, ldx, q, ldq, scale, amax, col_amax, st);
+  // longer rows: one workgroup per row, nchw = chunks per lane
+  if (col_amax) L8_REQUIRE(((uintptr_t)col_amax % 16) == 0, "l8_cast_rowwise: col_amax must be 16-byte aligned");
+  const int64_t nchw = (nch + kRowWaves - 1) / kRowWaves;
+  if (nchw <= 4) return launch_rowwise_wg<4>(x, R, C, ldx, q, ldq, scale, amax, col_amax, st);
+  if (nchw <= 6) return launch_rowwise_wg<6>(x, R, C, ldx, q, ldq, scale, amax, col_amax, st);
+  if (nchw <= 8) return launch_rowwise_wg<8>(x, R, C, ldx, q, ldq, scale, amax, col_amax, st);
+  if (nchw <= 16) return launch_rowwise_wg<16>(x, R, C, ldx, q, ldq, scale, amax, col_amax, st);
   int64_t blocks = R < (int64_t)num_cus() * 8 ? R : (int64_t)num_cus() * 8;
   hipLaunchKernelGGL(cast_rowwise_long_kernel, dim3((unsigned)blocks), dim3(kRowBlock), 0, st, (const uint16_t *)x, R,
                      (int)C, ldx, (uint8_t *)q, ldq, scale, (uint16_t *)amax, (uint32_t *)col_amax);
@@ -430,7 +599,7 @@ extern "C" int l8_col_amax(const void *x, int64_t R, int64_t C, int64_t ldx, flo
 
 extern "C" int l8_amax_reduce(const void *amax, int64_t n, void *amax_out, void *stream) {
   L8_REQUIRE(n >= 1 && amax && amax_out, "l8_amax_reduce: need n >= 1 and non-null pointers");
-  hipLaunchKernelGGL(amax_reduce_kernel, dim3(1), dim3(256), 0, (hipStream_t)stream, (const uint16_t *)amax, n,
+  hipLaunchKernelGGL(amax_reduce_kernel, dim3(1), dim3(1024), 0, (hipStream_t)stream, (const uint16_t *)amax, n,
                      (uint16_t *)amax_out);
   L8_HIP(hipGetLastError());
   return L8_OK;
@@ -438,8 +607,8 @@ extern "C" int l8_amax_reduce(const void *amax, int64_t n, void *amax_out, void 
 
 static int launch_transposed(bool per_col, const void *x, int64_t R, int64_t C, int64_t ldx, const void *amax,
                              const float *col_amax, void *q, int64_t ldq, float *scale, hipStream_t st) {
-  const int64_t gx = (C + kTC - 1) / kTC, gy = (R + kTR - 1) / kTR;
-  L8_REQUIRE(gy <= 65535, "transposed cast: R too large (%lld rows)", (long long)R);
+  const int64_t gx = ((C + kTC - 1) / kTC) * ((R + kTR - 1) / kTR), gy = 1;
+  L8_REQUIRE(gx < (1LL << 31), "transposed cast: shape too large (%lld x %lld)", (long long)R, (long long)C);
   const int vec = (ldq % 16 == 0 && aligned(q, 16)) ? 1 : 0;
   if (per_col)
     hipLaunchKernelGGL((cast_transposed_kernel<true>), dim3((unsigned)gx, (unsigned)gy), dim3(256), 0, st,

@@ -71,6 +71,9 @@ constexpr uint32_t kOOB = 0x80000000u;  // voffset that is out of range for ever
 #ifndef L8_GEMM_DIAG
 #define L8_GEMM_DIAG 0
 #endif
+#ifndef L8_STRADDLE
+#define L8_STRADDLE 2
+#endif
 
 // s_waitcnt for vmcnt <= n and lgkmcnt == 0 (expcnt untouched)
 #define L8_WAIT_VM_LGKM0(n) \
@@ -224,13 +227,15 @@ __global__ __launch_bounds__(WM *WN * 64) void gemm_nt_kernel(const GemmArgs p) 
 #pragma unroll
       for (int v = 0; v < 16; ++v) acc[tn][tm][v] = 0.0f;
 
-  auto mma = [&](v8i (&af)[TM], v8i (&bf)[TN]) {
+  // MFMAs lo .. hi-1 (of TM*TN) of one 64-byte step
+  auto mma = [&](v8i (&af)[TM], v8i (&bf)[TN], int lo, int hi) {
 #pragma unroll
     for (int tn = 0; tn < TN; ++tn)
 #pragma unroll
       for (int tm = 0; tm < TM; ++tm)
-        // D[i = n][j = m]: B rows feed the "A" port, A rows the "B" port
-        acc[tn][tm] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(bf[tn], af[tm], acc[tn][tm], 0, 0, 0, 0, 0, 0);
+        if (tn * TM + tm >= lo && tn * TM + tm < hi)
+          // D[i = n][j = m]: B rows feed the "A" port, A rows the "B" port
+          acc[tn][tm] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(bf[tn], af[tm], acc[tn][tm], 0, 0, 0, 0, 0, 0);
   };
 
   // prologue: R units in flight, K tile 0 published, its first half read
@@ -253,11 +258,12 @@ __global__ __launch_bounds__(WM *WN * 64) void gemm_nt_kernel(const GemmArgs p) 
   // A wave issues in order, so LDS reads and global loads are spread between
   // the MFMAs instead of queueing in front of them.
   constexpr int N_MMA = TM * TN, N_DSR = 2 * (TM + TN);
+  constexpr int STRADDLE = L8_STRADDLE < N_MMA - 2 ? L8_STRADDLE : 0;
   for (int kt = 0; kt < KT; ++kt) {
     if (L8_GEMM_DIAG != 2 && L8_GEMM_DIAG != 4) {
       read_frags(kt, 1, af1, bf1);
-      mma(af0, bf0);
-      interleave_step<N_MMA, N_DSR, 0, 0>();
+      mma(af0, bf0, 0, N_MMA - STRADDLE);
+      interleave_step<N_MMA - STRADDLE, N_DSR, 0, 0>();
     }
     __builtin_amdgcn_sched_barrier(0);
     L8_WAIT_VM_LGKM0(PEND);
@@ -269,8 +275,12 @@ __global__ __launch_bounds__(WM *WN * 64) void gemm_nt_kernel(const GemmArgs p) 
       issue_unit(2 * kt + R + 1);
     }
     if (L8_GEMM_DIAG != 2 && L8_GEMM_DIAG != 4) {
+      // the last MFMAs of the first half are issued after the barrier: they need
+      // registers only and keep the matrix cores busy while the waves regroup
+      mma(af0, bf0, N_MMA - STRADDLE, N_MMA);
+      __builtin_amdgcn_sched_barrier(0);
       read_frags(kt + 1, 0, af0, bf0);
-      mma(af1, bf1);
+      mma(af1, bf1, 0, N_MMA);
       interleave_step<N_MMA, N_DSR, (L8_GEMM_DIAG == 1 ? 0 : NA + NB), 0>();
     }
     __builtin_amdgcn_sched_barrier(0);
