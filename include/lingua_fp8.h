@@ -49,14 +49,18 @@ int l8_device_check(int device);
  *   q        e4m3fn [R,C], row stride ldq           (may be NULL: amax only)
  *   scale    fp32 [R] = max(f32(amax),1e-12)/448    (may be NULL with q)
  *   amax     bf16 [R] row amax, NaN propagating     (may be NULL)
- *   col_amax fp32 [C] (may be NULL): max-merged (atomically, as non-negative
- *            float bit patterns) with the column amaxes of x, so that a later
+ *   col_amax fp32 [C] (may be NULL): max-merged (as non-negative float bit
+ *            patterns) with the column amaxes of x, so that a later
  *            l8_cast_colwise_transposed() needs no pass of its own to find
  *            them.  The caller zero-fills it before the first merge.
+ *   workspace  device scratch of at least l8_cast_rowwise_workspace(R, C)
+ *            bytes, 16-byte aligned; needed only with col_amax (per-workgroup
+ *            partial maxima, folded by a second launch on the same stream).
  * Requires C % 8 == 0, ldx % 8 == 0, ldq % 8 == 0 and 16-byte aligned x / 8-byte aligned q. */
 int l8_cast_rowwise(const void *x, int64_t R, int64_t C, int64_t ldx,
                     void *q, int64_t ldq, float *scale, void *amax, float *col_amax,
-                    void *stream);
+                    void *workspace, int64_t workspace_bytes, void *stream);
+int64_t l8_cast_rowwise_workspace(int64_t R, int64_t C);
 
 /* Column amax on its own (same merge semantics as col_amax above). */
 int l8_col_amax(const void *x, int64_t R, int64_t C, int64_t ldx, float *col_amax, void *stream);

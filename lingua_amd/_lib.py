@@ -20,7 +20,8 @@ SIGNATURES = {
     "l8_version": [],
     "l8_last_error": [],
     "l8_device_check": [_int],
-    "l8_cast_rowwise": [_p, _i64, _i64, _i64, _p, _i64, _p, _p, _p, _p],
+    "l8_cast_rowwise": [_p, _i64, _i64, _i64, _p, _i64, _p, _p, _p, _p, _i64, _p],
+    "l8_cast_rowwise_workspace": [_i64, _i64],
     "l8_col_amax": [_p, _i64, _i64, _i64, _p, _p],
     "l8_amax_reduce": [_p, _i64, _p, _p],
     "l8_cast_tensorwise": [_p, _i64, _i64, _i64, _p, _int, _p, _i64, _p, _p],
@@ -30,6 +31,7 @@ SIGNATURES = {
     "l8_gemm_algo_name": [_int],
 }
 _RETURNS_STR = {"l8_last_error", "l8_gemm_algo_name"}
+_RETURNS_I64 = {"l8_cast_rowwise_workspace"}
 
 _lib = None
 _lock = threading.Lock()
@@ -52,7 +54,7 @@ def load():
             for name, argtypes in SIGNATURES.items():
                 fn = getattr(lib, name)
                 fn.argtypes = argtypes
-                fn.restype = ctypes.c_char_p if name in _RETURNS_STR else _int
+                fn.restype = ctypes.c_char_p if name in _RETURNS_STR else (_i64 if name in _RETURNS_I64 else _int)
             _lib = lib
     return _lib
 

@@ -13,8 +13,9 @@ namespace l8 {
 // between the amax reduction and the cast.  Lane l of chunk j holds columns
 // [j*512 + l*8, +8) (one 16-byte load, 1 KiB per wave instruction).
 // A workgroup is 4 waves; waves stride over rows so that the optional
-// column-amax by-product is accumulated in registers over many rows and merged
-// once per workgroup (LDS max, then one global atomic max per column).
+// column-amax by-product is accumulated in registers over many rows, merged
+// once per workgroup in LDS and written as one row of a partial-maxima array
+// that a small second kernel folds into the caller's column amaxes.
 // ---------------------------------------------------------------------------
 constexpr int kRowBlock = 256;
 constexpr int kRowWaves = kRowBlock / 64;
@@ -32,7 +33,7 @@ L8_DEV void load_row(v4i (&buf)[NCH], const uint16_t *row, int C, int lane) {
 template <int NCH, bool COLMAX>
 __global__ __launch_bounds__(kRowBlock, 2) void cast_rowwise_kernel(
     const uint16_t *__restrict__ x, int64_t R, int C, int64_t ldx, uint8_t *__restrict__ q, int64_t ldq,
-    float *__restrict__ scale, uint16_t *__restrict__ amax_out, uint32_t *__restrict__ col_amax) {
+    float *__restrict__ scale, uint16_t *__restrict__ amax_out, uint16_t *__restrict__ col_partials) {
   extern __shared__ uint32_t lds_colmax[];  // [C/2] packed bf16 pairs when COLMAX
   // the next row is prefetched into a second register set unless that would
   // push the wave beyond 256 VGPRs (two waves per SIMD are worth more)
@@ -108,10 +109,9 @@ __global__ __launch_bounds__(kRowBlock, 2) void cast_rowwise_kernel(
 
   if (COLMAX) {
     // merge the four waves' column maxima through LDS, one wave after the other
-    // (packed pairs, plain reads and writes), then raise the global values:
-    // a plain read first, the atomic only where this workgroup has a larger
-    // value -- late workgroups rarely do, so atomics stay rare.  A stale read
-    // can only cause a redundant atomic, never a missed one.
+    // (packed pairs, plain reads and writes), then write this workgroup's row of
+    // the partial-maxima array; a second small kernel folds the rows.  (Global
+    // atomics from every workgroup cost more than the cast itself.)
     v4i *lds4 = (v4i *)lds_colmax;
     for (int w = 0; w < kRowWaves; ++w) {
       if (wave == w) {
@@ -125,19 +125,12 @@ __global__ __launch_bounds__(kRowBlock, 2) void cast_rowwise_kernel(
 #pragma unroll
               for (int k = 0; k < 4; ++k) mine[k] = (int)pk_absmax_u16((uint32_t)old[k], (uint32_t)mine[k]);
             }
-            lds4[c / 8] = mine;
+            if (w == kRowWaves - 1) *(v4i *)(col_partials + (int64_t)blockIdx.x * C + c) = mine;
+            else lds4[c / 8] = mine;
           }
         }
       }
       __syncthreads();
-    }
-    for (int i = threadIdx.x; i < C / 2; i += kRowBlock) {
-      const uint32_t v = lds_colmax[i];
-      const uint32_t lo = (v & 0xffffu) << 16, hi = v & 0xffff0000u;  // bf16 -> fp32 bit patterns
-      const uint32_t g0 = __builtin_nontemporal_load(&col_amax[2 * i]);
-      const uint32_t g1 = __builtin_nontemporal_load(&col_amax[2 * i + 1]);
-      if (lo > g0) atomicMax(&col_amax[2 * i], lo);
-      if (hi > g1) atomicMax(&col_amax[2 * i + 1], hi);
     }
   }
 }
@@ -150,7 +143,7 @@ __global__ __launch_bounds__(kRowBlock, 2) void cast_rowwise_kernel(
 template <int NCHW, bool COLMAX>
 __global__ __launch_bounds__(kRowBlock, (NCHW <= 4 ? 4 : (NCHW <= 8 ? 2 : 1))) void cast_rowwise_wg_kernel(
     const uint16_t *__restrict__ x, int64_t R, int C, int64_t ldx, uint8_t *__restrict__ q, int64_t ldq,
-    float *__restrict__ scale, uint16_t *__restrict__ amax_out, uint32_t *__restrict__ col_amax) {
+    float *__restrict__ scale, uint16_t *__restrict__ amax_out, uint16_t *__restrict__ col_partials) {
   __shared__ uint32_t red[2][kRowWaves];
   const int lane = threadIdx.x & 63;
   const int wave = threadIdx.x >> 6;
@@ -213,26 +206,31 @@ __global__ __launch_bounds__(kRowBlock, (NCHW <= 4 ? 4 : (NCHW <= 8 ? 2 : 1))) v
     r = rn;
   }
   if (COLMAX) {
-    // plain read first, atomic only where this workgroup has a larger value (a
-    // stale read can only cause a redundant atomic, never a missed one)
+    // the four waves own disjoint columns: together they write this workgroup's
+    // row of the partial-maxima array
 #pragma unroll
     for (int j = 0; j < NCHW; ++j) {
       const int c = col_of(j);
-      if (c < C) {
-        const v4i g0 = __builtin_nontemporal_load((const v4i *)(col_amax + c));
-        const v4i g1 = __builtin_nontemporal_load((const v4i *)(col_amax + c + 4));
-#pragma unroll
-        for (int k = 0; k < 4; ++k) {
-          const uint32_t v = cmax[j * 4 + k];
-          const uint32_t lo = (v & 0xffffu) << 16, hi = v & 0xffff0000u;
-          const uint32_t glo = (uint32_t)(k < 2 ? g0[2 * k] : g1[2 * k - 4]);
-          const uint32_t ghi = (uint32_t)(k < 2 ? g0[2 * k + 1] : g1[2 * k - 3]);
-          if (lo > glo) atomicMax(&col_amax[c + 2 * k], lo);
-          if (hi > ghi) atomicMax(&col_amax[c + 2 * k + 1], hi);
-        }
-      }
+      if (c < C)
+        *(v4i *)(col_partials + (int64_t)blockIdx.x * C + c) =
+            v4i{(int)cmax[j * 4], (int)cmax[j * 4 + 1], (int)cmax[j * 4 + 2], (int)cmax[j * 4 + 3]};
     }
   }
+}
+
+// Folds the partial column maxima [n_slots, C] (bf16) into col_amax[C] (fp32 bit
+// patterns, max-merged).  Thread (x, y): column pair x, slots y*32 .. y*32+31.
+__global__ __launch_bounds__(256) void colmax_fold_kernel(const uint16_t *__restrict__ partials, int n_slots, int C,
+                                                          uint32_t *__restrict__ col_amax) {
+  const int pair = blockIdx.x * 256 + threadIdx.x;
+  if (pair * 2 >= C) return;
+  const int s0 = blockIdx.y * 32, s1 = (s0 + 32 < n_slots) ? s0 + 32 : n_slots;
+  uint32_t m = 0;
+  for (int sl = s0; sl < s1; ++sl)
+    m = pk_absmax_u16(m, __builtin_nontemporal_load((const uint32_t *)(partials + (int64_t)sl * C) + pair));
+  const uint32_t lo = (m & 0xffffu) << 16, hi = m & 0xffff0000u;  // bf16 -> fp32 bit patterns
+  if (lo) atomicMax(&col_amax[2 * pair], lo);
+  if (hi) atomicMax(&col_amax[2 * pair + 1], hi);
 }
 
 // Fallback for rows too long to keep in registers: two passes over the row by
@@ -502,42 +500,60 @@ __global__ __launch_bounds__(256) void cast_transposed_kernel(
 // ---------------------------------------------------------------------------
 // host entry points
 // ---------------------------------------------------------------------------
+static bool aligned(const void *p, size_t a) { return ((uintptr_t)p % a) == 0; }
+
+// Number of workgroups (= rows of the partial-maxima workspace) of the two
+// register-resident row-wise kernels; 0 when the shape uses the two-pass kernel.
+static int64_t rowwise_blocks(int64_t R, int64_t C, bool colmax) {
+  const int64_t nch = (C + 511) / 512;
+  const int64_t cus = num_cus();
+  if (nch <= 8) {
+    const int64_t blocks = (R + kRowWaves - 1) / kRowWaves, cap = cus * (colmax ? 2 : 8);
+    return blocks < cap ? blocks : cap;
+  }
+  if ((nch + kRowWaves - 1) / kRowWaves <= 16) {
+    const int64_t cap = cus * (colmax ? 2 : 8);
+    return R < cap ? R : cap;
+  }
+  return 0;
+}
+
+static int fold_colmax(const void *partials, int64_t slots, int64_t C, float *col_amax, hipStream_t st) {
+  hipLaunchKernelGGL(colmax_fold_kernel, dim3((unsigned)((C / 2 + 255) / 256), (unsigned)((slots + 31) / 32)), dim3(256), 0,
+                     st, (const uint16_t *)partials, (int)slots, (int)C, (uint32_t *)col_amax);
+  L8_HIP(hipGetLastError());
+  return L8_OK;
+}
+
 template <int NCH>
 static int launch_rowwise(const void *x, int64_t R, int64_t C, int64_t ldx, void *q, int64_t ldq, float *scale,
-                          void *amax, float *col_amax, hipStream_t st) {
-  const int cus = num_cus();
-  int64_t blocks = (R + kRowWaves - 1) / kRowWaves;
-  // with the column-amax by-product fewer, longer-lived workgroups mean fewer merges
-  const int64_t cap = (int64_t)cus * (col_amax ? 2 : 8);
-  if (blocks > cap) blocks = cap;
+                          void *amax, float *col_amax, void *ws, hipStream_t st) {
+  const int64_t blocks = rowwise_blocks(R, C, col_amax != nullptr);
   if (col_amax) {
     const size_t lds = (size_t)C * sizeof(uint16_t);
     hipLaunchKernelGGL((cast_rowwise_kernel<NCH, true>), dim3((unsigned)blocks), dim3(kRowBlock), lds, st,
-                       (const uint16_t *)x, R, (int)C, ldx, (uint8_t *)q, ldq, scale, (uint16_t *)amax,
-                       (uint32_t *)col_amax);
-  } else {
-    hipLaunchKernelGGL((cast_rowwise_kernel<NCH, false>), dim3((unsigned)blocks), dim3(kRowBlock), 0, st,
-                       (const uint16_t *)x, R, (int)C, ldx, (uint8_t *)q, ldq, scale, (uint16_t *)amax,
-                       (uint32_t *)nullptr);
+                       (const uint16_t *)x, R, (int)C, ldx, (uint8_t *)q, ldq, scale, (uint16_t *)amax, (uint16_t *)ws);
+    L8_HIP(hipGetLastError());
+    return fold_colmax(ws, blocks, C, col_amax, st);
   }
+  hipLaunchKernelGGL((cast_rowwise_kernel<NCH, false>), dim3((unsigned)blocks), dim3(kRowBlock), 0, st,
+                     (const uint16_t *)x, R, (int)C, ldx, (uint8_t *)q, ldq, scale, (uint16_t *)amax, (uint16_t *)nullptr);
   L8_HIP(hipGetLastError());
   return L8_OK;
 }
 
 template <int NCHW>
 static int launch_rowwise_wg(const void *x, int64_t R, int64_t C, int64_t ldx, void *q, int64_t ldq, float *scale,
-                             void *amax, float *col_amax, hipStream_t st) {
-  int64_t blocks = R;
-  const int64_t cap = (int64_t)num_cus() * (col_amax ? 4 : 8);
-  if (blocks > cap) blocks = cap;
-  if (col_amax)
+                             void *amax, float *col_amax, void *ws, hipStream_t st) {
+  const int64_t blocks = rowwise_blocks(R, C, col_amax != nullptr);
+  if (col_amax) {
     hipLaunchKernelGGL((cast_rowwise_wg_kernel<NCHW, true>), dim3((unsigned)blocks), dim3(kRowBlock), 0, st,
-                       (const uint16_t *)x, R, (int)C, ldx, (uint8_t *)q, ldq, scale, (uint16_t *)amax,
-                       (uint32_t *)col_amax);
-  else
-    hipLaunchKernelGGL((cast_rowwise_wg_kernel<NCHW, false>), dim3((unsigned)blocks), dim3(kRowBlock), 0, st,
-                       (const uint16_t *)x, R, (int)C, ldx, (uint8_t *)q, ldq, scale, (uint16_t *)amax,
-                       (uint32_t *)nullptr);
+                       (const uint16_t *)x, R, (int)C, ldx, (uint8_t *)q, ldq, scale, (uint16_t *)amax, (uint16_t *)ws);
+    L8_HIP(hipGetLastError());
+    return fold_colmax(ws, blocks, C, col_amax, st);
+  }
+  hipLaunchKernelGGL((cast_rowwise_wg_kernel<NCHW, false>), dim3((unsigned)blocks), dim3(kRowBlock), 0, st,
+                     (const uint16_t *)x, R, (int)C, ldx, (uint8_t *)q, ldq, scale, (uint16_t *)amax, (uint16_t *)nullptr);
   L8_HIP(hipGetLastError());
   return L8_OK;
 }
@@ -546,10 +562,14 @@ static int launch_rowwise_wg(const void *x, int64_t R, int64_t C, int64_t ldx, v
 
 using namespace l8;
 
-static bool aligned(const void *p, size_t a) { return ((uintptr_t)p % a) == 0; }
+
+extern "C" int64_t l8_cast_rowwise_workspace(int64_t R, int64_t C) {
+  if (R <= 0 || C <= 0) return 0;
+  return rowwise_blocks(R, C, true) * C * (int64_t)sizeof(uint16_t);
+}
 
 extern "C" int l8_cast_rowwise(const void *x, int64_t R, int64_t C, int64_t ldx, void *q, int64_t ldq, float *scale,
-                               void *amax, float *col_amax, void *stream) {
+                               void *amax, float *col_amax, void *workspace, int64_t workspace_bytes, void *stream) {
   L8_REQUIRE(R >= 0 && C >= 0, "l8_cast_rowwise: negative shape R=%lld C=%lld", (long long)R, (long long)C);
   if (R == 0 || C == 0) return L8_OK;
   L8_REQUIRE(x != nullptr, "l8_cast_rowwise: x is null");
@@ -559,17 +579,23 @@ extern "C" int l8_cast_rowwise(const void *x, int64_t R, int64_t C, int64_t ldx,
   L8_REQUIRE(aligned(x, 16), "l8_cast_rowwise: x must be 16-byte aligned");
   if (q) L8_REQUIRE(ldq % 8 == 0 && ldq >= C && aligned(q, 8), "l8_cast_rowwise: q must be 8-byte aligned with ldq %% 8 == 0, ldq >= C");
   L8_REQUIRE(C < (1LL << 31), "l8_cast_rowwise: C too large");
+  if (col_amax) {
+    const int64_t need = l8_cast_rowwise_workspace(R, C);
+    L8_REQUIRE(need == 0 || (workspace != nullptr && workspace_bytes >= need && aligned(workspace, 16)),
+               "l8_cast_rowwise: col_amax needs a 16-byte aligned workspace of %lld bytes (l8_cast_rowwise_workspace)",
+               (long long)need);
+  }
   hipStream_t st = (hipStream_t)stream;
+  void *ws = workspace;
   const int64_t nch = (C + 511) / 512;
-  if (nch <= 4) return launch_rowwise<4>(x, R, C, ldx, q, ldq, scale, amax, col_amax, st);
-  if (nch <= 8) return launch_rowwise<8>(x, R, C, ldx, q, ldq, scale, amax, col_amax, st);
+  if (nch <= 4) return launch_rowwise<4>(x, R, C, ldx, q, ldq, scale, amax, col_amax, ws, st);
+  if (nch <= 8) return launch_rowwise<8>(x, R, C, ldx, q, ldq, scale, amax, col_amax, ws, st);
   // longer rows: one workgroup per row, nchw = chunks per lane
-  if (col_amax) L8_REQUIRE(((uintptr_t)col_amax % 16) == 0, "l8_cast_rowwise: col_amax must be 16-byte aligned");
   const int64_t nchw = (nch + kRowWaves - 1) / kRowWaves;
-  if (nchw <= 4) return launch_rowwise_wg<4>(x, R, C, ldx, q, ldq, scale, amax, col_amax, st);
-  if (nchw <= 6) return launch_rowwise_wg<6>(x, R, C, ldx, q, ldq, scale, amax, col_amax, st);
-  if (nchw <= 8) return launch_rowwise_wg<8>(x, R, C, ldx, q, ldq, scale, amax, col_amax, st);
-  if (nchw <= 16) return launch_rowwise_wg<16>(x, R, C, ldx, q, ldq, scale, amax, col_amax, st);
+  if (nchw <= 4) return launch_rowwise_wg<4>(x, R, C, ldx, q, ldq, scale, amax, col_amax, ws, st);
+  if (nchw <= 6) return launch_rowwise_wg<6>(x, R, C, ldx, q, ldq, scale, amax, col_amax, ws, st);
+  if (nchw <= 8) return launch_rowwise_wg<8>(x, R, C, ldx, q, ldq, scale, amax, col_amax, ws, st);
+  if (nchw <= 16) return launch_rowwise_wg<16>(x, R, C, ldx, q, ldq, scale, amax, col_amax, ws, st);
   int64_t blocks = R < (int64_t)num_cus() * 8 ? R : (int64_t)num_cus() * 8;
   hipLaunchKernelGGL(cast_rowwise_long_kernel, dim3((unsigned)blocks), dim3(kRowBlock), 0, st, (const uint16_t *)x, R,
                      (int)C, ldx, (uint8_t *)q, ldq, scale, (uint16_t *)amax, (uint32_t *)col_amax);

@@ -71,10 +71,16 @@ def cast_rowwise(x: torch.Tensor, col_amax: Optional[torch.Tensor] = None, want_
     amax = torch.empty((R, 1), dtype=torch.bfloat16, device=x.device)
     if col_amax is not None and (col_amax.dtype != torch.float32 or col_amax.numel() != C or not col_amax.is_contiguous()):
         raise RuntimeError("cast_rowwise: col_amax must be a contiguous fp32 tensor with C elements")
+    ws, ws_bytes = None, 0
+    if col_amax is not None:
+        ws_bytes = _lib.load().l8_cast_rowwise_workspace(R, C)
+        if ws_bytes:
+            ws = torch.empty(ws_bytes, dtype=torch.uint8, device=x.device)
     with _timed("cast_rowwise", R * C * (3 if want_q else 2) + 4 * R + (4 * C if col_amax is not None else 0), x.device):
         code = _lib.load().l8_cast_rowwise(
             x.data_ptr(), R, C, _ld(x), q.data_ptr() if want_q else None, C, scale.data_ptr(), amax.data_ptr(),
-            col_amax.data_ptr() if col_amax is not None else None, st)
+            col_amax.data_ptr() if col_amax is not None else None, ws.data_ptr() if ws is not None else None,
+            ws_bytes, st)
     _lib.check(code, "l8_cast_rowwise")
     return q, scale, amax
 

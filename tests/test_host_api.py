@@ -21,7 +21,7 @@ def test_library_exports_every_declared_symbol():
     header = re.sub(r"/\*.*?\*/", "", header, flags=re.S)
     declared = set(re.findall(r"\b(l8_\w+)\s*\(", header))
     assert {"l8_cast_rowwise", "l8_cast_tensorwise", "l8_cast_colwise_transposed", "l8_gemm_nt", "l8_col_amax",
-            "l8_amax_reduce", "l8_version", "l8_last_error", "l8_device_check"} <= declared
+            "l8_amax_reduce", "l8_version", "l8_last_error", "l8_device_check", "l8_cast_rowwise_workspace"} <= declared
     lib = ctypes.CDLL(_lib.LIB_PATH)
     for name in declared:
         assert hasattr(lib, name), name
@@ -38,12 +38,16 @@ def test_argument_validation_happens_before_launch():
     assert lib.l8_gemm_nt(fake, fake, 4, 4, 16, 16, 16, fake, 1, fake, 1, None, fake, 4, 99, None) == -1
     assert lib.l8_gemm_nt(None, fake, 4, 4, 16, 16, 16, fake, 1, fake, 1, None, fake, 4, 0, None) == -1
     assert lib.l8_gemm_nt(fake + 1, fake, 4, 4, 16, 16, 16, fake, 1, fake, 1, None, fake, 4, 0, None) == -1
-    assert lib.l8_cast_rowwise(fake, 4, 12, 12, fake, 12, fake, None, None, None) == -1
-    assert lib.l8_cast_rowwise(fake, -1, 8, 8, fake, 8, fake, None, None, None) == -1
+    assert lib.l8_cast_rowwise(fake, 4, 12, 12, fake, 12, fake, None, None, None, 0, None) == -1
+    assert lib.l8_cast_rowwise(fake, -1, 8, 8, fake, 8, fake, None, None, None, 0, None) == -1
     assert lib.l8_cast_tensorwise(fake, 4, 8, 8, None, 0, fake, 8, fake, None) == -1
     assert lib.l8_cast_colwise_transposed(fake, 4, 8, 8, None, fake, 4, fake, None) == -1
     # empty problems are accepted and do nothing
-    assert lib.l8_cast_rowwise(None, 0, 8, 8, None, 8, None, None, None, None) == 0
+    assert lib.l8_cast_rowwise(None, 0, 8, 8, None, 8, None, None, None, None, 0, None) == 0
+    # the column-amax by-product needs the workspace the library asks for
+    assert lib.l8_cast_rowwise_workspace(64, 1024) > 0
+    assert lib.l8_cast_rowwise(fake, 64, 1024, 1024, fake, 1024, fake, None, fake, None, 0, None) == -1
+    assert "workspace" in _lib.last_error()
     assert lib.l8_gemm_nt(None, None, 0, 4, 16, 16, 16, None, 1, None, 1, None, None, 4, 0, None) == 0
 
 
