@@ -21,8 +21,13 @@
 //     (`s_waitcnt vmcnt(n)`), one barrier per K tile;
 //   * fragments are software-pipelined through two register sets: each half
 //     of a trip runs the MFMAs of one 64-byte step while the next step is
-//     read from LDS, and the instruction order interleaves MFMAs, LDS reads
-//     and global loads (a wave issues in order);
+//     read from LDS.  A wave issues in order, so the instruction stream is
+//     laid out by hand as groups of one MFMA + its share of the LDS reads +
+//     its share of the panel loads, with scheduling fences between groups:
+//     one unit is requested during each half of a trip.  (Requesting both
+//     units in a burst after the barrier left the waves queueing at the
+//     vector-memory port with idle matrix cores: 2830 -> 2310 shader clocks
+//     per trip, the matrix cores alone need 2048.);
 //   * LDS rows are 128 bytes (8 chunks of 16 B); chunk c of row r lives at
 //     position c ^ f(r), f(r) = (r & 7) ^ ((r >> 3) & 1): the 16-byte
 //     fragment reads of any 16 consecutive rows then cover all 64 banks once
@@ -79,24 +84,7 @@ constexpr uint32_t kOOB = 0x80000000u;  // voffset that is out of range for ever
 #define L8_WAIT_VM_LGKM0(n) \
   __builtin_amdgcn_s_waitcnt(((n) & 0xF) | (0x7 << 4) | (0x0 << 8) | ((((n) >> 4) & 0x3) << 14))
 
-#if defined(__HIP_DEVICE_COMPILE__)
-// Scheduling recipe for one half trip: N_MMA groups of "one MFMA, then a share
-// of the N_DSR LDS reads (spread over the first N_MMA-2 groups), then one of
-// the N_VMEM global loads".  The group sizes must be literals, hence the recursion.
-template <int N_MMA, int N_DSR, int N_VMEM, int I>
-L8_DEV void interleave_step() {
-  if constexpr (I < N_MMA) {
-    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-    constexpr int slots = N_MMA > 2 ? N_MMA - 2 : 1;
-    constexpr int r0 = (N_DSR * I) / slots, r1 = (N_DSR * (I + 1)) / slots;
-    if constexpr (I < slots && r1 > r0) __builtin_amdgcn_sched_group_barrier(0x100, r1 - r0, 0);
-    if constexpr (I < N_VMEM) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
-    interleave_step<N_MMA, N_DSR, N_VMEM, I + 1>();
-  }
-}
-#endif
-
-template <int WM, int WN, int TM, int TN, int R, int GROUP_M>
+template <int WM, int WN, int TM, int TN, int R, int GROUP_M, int PF>
 __global__ __launch_bounds__(WM *WN * 64) void gemm_nt_kernel(const GemmArgs p) {
 #if defined(__HIP_DEVICE_COMPILE__)
   constexpr int BM = WM * TM * 32, BN = WN * TN * 32, BK = 128;
@@ -105,11 +93,14 @@ __global__ __launch_bounds__(WM *WN * 64) void gemm_nt_kernel(const GemmArgs p) 
   constexpr int UNIT = A_BYTES > B_BYTES ? A_BYTES : B_BYTES;  // one ring slot holds an A or a B panel of one K tile
   static_assert((BM / 8) % NW == 0 && (BN / 8) % NW == 0, "tile rows must split evenly over waves");
   constexpr int NA = BM / 8 / NW, NB = BN / 8 / NW;  // 1 KiB wave loads (8 rows x 128 B) per panel per wave
+  // L2 touches (PF > 0): one lane per panel row, every wave covers 64 rows per instruction
+  constexpr int PFA = PF > 0 ? (BM + NW * 64 - 1) / (NW * 64) : 0, PFB = PF > 0 ? (BN + NW * 64 - 1) / (NW * 64) : 0;
+  constexpr int IA = NA + PFA, IB = NB + PFB;  // vector-memory instructions per unit per wave
   // loads of the units that may still be in flight when a K tile is published:
   // the ring holds the tile being read (2 slots), the tile being published (2
   // slots) and R-4 younger units, the first of which is an A panel
-  constexpr int PEND = ((R - 4 + 1) / 2) * NA + ((R - 4) / 2) * NB;
-  constexpr int PEND0 = ((R - 2 + 1) / 2) * NA + ((R - 2) / 2) * NB;  // same for the prologue (R-2 younger units)
+  constexpr int PEND = ((R - 4 + 1) / 2) * IA + ((R - 4) / 2) * IB;
+  constexpr int PEND0 = ((R - 3 + 1) / 2) * IA + ((R - 3) / 2) * IB;  // same for the prologue (R-3 younger units)
   static_assert(R >= 4 && PEND0 <= 63, "vmcnt is a 6-bit counter");
   extern __shared__ __attribute__((aligned(1024))) uint8_t smem[];
 
@@ -118,7 +109,7 @@ __global__ __launch_bounds__(WM *WN * 64) void gemm_nt_kernel(const GemmArgs p) 
   const int wm = wave / WN, wn = wave % WN;
 
   // ---- XCD-aware, grouped workgroup -> tile mapping ----
-  int tile_m, tile_n;
+  int tile_m, tile_n, row_in_group;
   {
     const int nb = p.tiles_m * p.tiles_n;
     const int pid = blockIdx.x;
@@ -130,7 +121,8 @@ __global__ __launch_bounds__(WM *WN * 64) void gemm_nt_kernel(const GemmArgs p) 
     const int first_m = grp * GROUP_M;
     const int gsz = (p.tiles_m - first_m < GROUP_M) ? p.tiles_m - first_m : GROUP_M;
     const int in_grp = lin - grp * per_group;
-    tile_m = first_m + in_grp % gsz;
+    row_in_group = in_grp % gsz;
+    tile_m = first_m + row_in_group;
     tile_n = in_grp / gsz;
   }
   if (L8_GEMM_DIAG == 4) { tile_m = 0; tile_n = 0; }
@@ -147,54 +139,78 @@ __global__ __launch_bounds__(WM *WN * 64) void gemm_nt_kernel(const GemmArgs p) 
   const __amdgpu_buffer_rsrc_t rsA = make_rsrc(Ablk, a_left < 0x7fffffff ? (uint32_t)a_left : 0x7fffffffu);
   const __amdgpu_buffer_rsrc_t rsB = make_rsrc(Bblk, b_left < 0x7fffffff ? (uint32_t)b_left : 0x7fffffffu);
 
-  uint32_t a_voff[NA], b_voff[NB];
+  // Wave load j of a panel covers the 8 rows of group g = wave * N + j.  The
+  // per-lane part of the address depends on the parity of g only (N is even, so
+  // on the parity of j); the rest is scalar.  Rows beyond M / N need no test:
+  // their offsets lie beyond the resource's range.
+  static_assert(NA % 2 == 0 && NB % 2 == 0, "wave loads per panel must be even");
+  const uint32_t a_voff[2] = {(uint32_t)(lrow * (int)p.lda + (lpos ^ lrow) * 16), (uint32_t)(lrow * (int)p.lda + (lpos ^ lrow ^ 1) * 16)};
+  const uint32_t b_voff[2] = {(uint32_t)(lrow * (int)p.ldb + (lpos ^ lrow) * 16), (uint32_t)(lrow * (int)p.ldb + (lpos ^ lrow ^ 1) * 16)};
+  const int a_lda8 = 8 * (int)p.lda, b_ldb8 = 8 * (int)p.ldb;
+  const int a_srow = wave * NA * a_lda8, b_srow = wave * NB * b_ldb8;
+  // L2 touches.  The 32 workgroups resident on an XCD form a GROUP_M x (32 / GROUP_M)
+  // block of tiles: 32 / GROUP_M of them stream the same A panel and GROUP_M the
+  // same B panel.  Each workgroup touches (one dword per 128-byte line) only its
+  // share of the rows of the K tile PF trips ahead, so that the line is in the
+  // XCD's L2 when the panel loads of all the sharers ask for it.
+  uint32_t pfa_voff[PFA > 0 ? PFA : 1], pfb_voff[PFB > 0 ? PFB : 1];
+  if constexpr (PF > 0) {
+    constexpr int SA = 32 / GROUP_M >= 1 ? 32 / GROUP_M : 1, SB = GROUP_M;
+    const int slice_a = tile_n % SA, slice_b = row_in_group % SB;
 #pragma unroll
-  for (int i = 0; i < NA; ++i) {
-    const int g = wave * NA + i, row = g * 8 + lrow;
-    const int chunk = lpos ^ lrow ^ (g & 1);
-    a_voff[i] = (m0 + row < p.M) ? (uint32_t)(row * (int)p.lda + chunk * 16) : kOOB;
-  }
+    for (int i = 0; i < PFA; ++i) {
+      const int row = (i * NW + wave) * 64 + lane;
+      pfa_voff[i] = (row < BM && row % SA == slice_a && m0 + row < p.M) ? (uint32_t)(row * (int)p.lda) : kOOB;
+    }
 #pragma unroll
-  for (int i = 0; i < NB; ++i) {
-    const int g = wave * NB + i, row = g * 8 + lrow;
-    const int chunk = lpos ^ lrow ^ (g & 1);
-    b_voff[i] = (n0 + row < p.N) ? (uint32_t)(row * (int)p.ldb + chunk * 16) : kOOB;
+    for (int i = 0; i < PFB; ++i) {
+      const int row = (i * NW + wave) * 64 + lane;
+      pfb_voff[i] = (row < BN && row % SB == slice_b && n0 + row < p.N) ? (uint32_t)(row * (int)p.ldb) : kOOB;
+    }
   }
   const int chunk_even = (lpos ^ lrow) * 16, chunk_odd = (lpos ^ lrow ^ 1) * 16;  // byte offset in the row, by parity of g
 
   const int KT = (p.K + BK - 1) / BK;
+  const uint32_t lds0 = (uint32_t)(uintptr_t)(lds_ptr_t)smem;
+  auto wrap = [](int slot) { return slot >= R ? slot - R : slot; };  // slot in [0, 2R)
   // Units are issued in the order A(0), B(0), A(1), B(1), ...; unit u lives in
-  // ring slot u % R.  Every call issues the full count of loads so that the
-  // vmcnt arithmetic is uniform; K tiles at or beyond the end, rows beyond
-  // M / N and chunks beyond K use an out-of-range offset, which the buffer unit
-  // turns into zeros in LDS.
-  auto issue_a = [&](int kt) {
+  // ring slot u % R (the callers keep the slot numbers as running scalars).
+  // Every unit issues its full count of loads so that the vmcnt arithmetic is
+  // uniform; K tiles at or beyond the end, rows beyond M / N and chunks beyond
+  // K use an out-of-range offset, which the buffer unit turns into zeros in LDS.
+  // load_one: i-th vector-memory instruction (of IA or IB) of the unit of K
+  // tile kt (A or B panel) into ring slot `slot`: first the L2 touches, then
+  // the 1 KiB panel loads.
+  auto load_one = [&](bool is_b, int kt, int slot, int i) {
     const int k0 = kt * BK;
-    uint8_t *dst = smem + ((2 * kt) % R) * UNIT + wave * (NA * 1024);
     const uint32_t m_even = (k0 + chunk_even < p.K) ? 0u : kOOB, m_odd = (k0 + chunk_odd < p.K) ? 0u : kOOB;
-#pragma unroll
-    for (int i = 0; i < NA; ++i)
-      __builtin_amdgcn_raw_ptr_buffer_load_lds(rsA, (lds_ptr_t)(dst + i * 1024), 16,
-                                               a_voff[i] | (((wave * NA + i) & 1) ? m_odd : m_even), k0, 0, 0);
-  };
-  auto issue_b = [&](int kt) {
-    const int k0 = kt * BK;
-    uint8_t *dst = smem + ((2 * kt + 1) % R) * UNIT + wave * (NB * 1024);
-    const uint32_t m_even = (k0 + chunk_even < p.K) ? 0u : kOOB, m_odd = (k0 + chunk_odd < p.K) ? 0u : kOOB;
-#pragma unroll
-    for (int i = 0; i < NB; ++i)
-      __builtin_amdgcn_raw_ptr_buffer_load_lds(rsB, (lds_ptr_t)(dst + i * 1024), 16,
-                                               b_voff[i] | (((wave * NB + i) & 1) ? m_odd : m_even), k0, 0, 0);
-  };
-  auto issue_unit = [&](int u) {
-    if (u & 1) issue_b(u >> 1);
-    else issue_a(u >> 1);
+    if (!is_b) {
+      const uint32_t dst = lds0 + slot * UNIT + wave * (NA * 1024);
+      // a touched dword lands in this wave's own part of the slot and is
+      // overwritten by the panel loads that follow (a wave's loads return in order)
+      if (i < PFA)
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(rsA, reinterpret_cast<lds_ptr_t>(dst), 4,
+                                                 pfa_voff[i < PFA ? i : 0] | ((k0 + PF * BK < p.K) ? 0u : kOOB), k0 + PF * BK, 0, 0);
+      else
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(rsA, reinterpret_cast<lds_ptr_t>(dst + (i - PFA) * 1024), 16,
+                                                 a_voff[(i - PFA) & 1] | (((i - PFA) & 1) ? m_odd : m_even),
+                                                 k0 + a_srow + (i - PFA) * a_lda8, 0, 0);
+    } else {
+      const uint32_t dst = lds0 + slot * UNIT + wave * (NB * 1024);
+      if (i < PFB)
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(rsB, reinterpret_cast<lds_ptr_t>(dst), 4,
+                                                 pfb_voff[i < PFB ? i : 0] | ((k0 + PF * BK < p.K) ? 0u : kOOB), k0 + PF * BK, 0, 0);
+      else
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(rsB, reinterpret_cast<lds_ptr_t>(dst + (i - PFB) * 1024), 16,
+                                                 b_voff[(i - PFB) & 1] | (((i - PFB) & 1) ? m_odd : m_even),
+                                                 k0 + b_srow + (i - PFB) * b_ldb8, 0, 0);
+    }
   };
 
   // ---- LDS -> register fragment plan ----
   const int l31 = lane & 31, h = lane >> 5;
   const int fr = (l31 & 7) ^ ((l31 >> 3) & 1);
-  int foff[2][2];
+  uint32_t foff[2][2];
 #pragma unroll
   for (int s = 0; s < 2; ++s)
 #pragma unroll
@@ -202,21 +218,27 @@ __global__ __launch_bounds__(WM *WN * 64) void gemm_nt_kernel(const GemmArgs p) 
   const int a_base = wm * (TM * 32 * BK);
   const int b_base = wn * (TN * 32 * BK);
 
-  auto read_frags = [&](int kt, int s, v8i (&af)[TM], v8i (&bf)[TN]) {
-    const uint8_t *pa = smem + ((2 * kt) % R) * UNIT + a_base;
-    const uint8_t *pb = smem + ((2 * kt + 1) % R) * UNIT + b_base;
-#pragma unroll
-    for (int tm = 0; tm < TM; ++tm) {
-      const v4i lo = *(const v4i *)(pa + tm * (32 * BK) + foff[s][0]);
-      const v4i hi = *(const v4i *)(pa + tm * (32 * BK) + foff[s][1]);
-      af[tm] = v8i{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
-    }
-#pragma unroll
-    for (int tn = 0; tn < TN; ++tn) {
-      const v4i lo = *(const v4i *)(pb + tn * (32 * BK) + foff[s][0]);
-      const v4i hi = *(const v4i *)(pb + tn * (32 * BK) + foff[s][1]);
-      bf[tn] = v8i{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
-    }
+  // LDS addresses of the two 16-byte pieces a lane reads of its row, for step s
+  // of the K tile whose panels sit in slots slot_a / slot_b.  The additions are
+  // opaque to the compiler on purpose: it would otherwise keep a register per
+  // (slot, piece) combination alive across the loop.
+  typedef const __attribute__((address_space(3))) v4i *lds_v4i_ptr;
+  auto frag_addrs = [&](int slot_a, int slot_b, int s, uint32_t (&ad)[4]) {
+    const uint32_t sa = lds0 + slot_a * UNIT + a_base, sb = lds0 + slot_b * UNIT + b_base;
+    asm volatile("v_add_u32 %0, %1, %2" : "=v"(ad[0]) : "s"(sa), "v"(foff[s][0]));
+    asm volatile("v_add_u32 %0, %1, %2" : "=v"(ad[1]) : "s"(sa), "v"(foff[s][1]));
+    asm volatile("v_add_u32 %0, %1, %2" : "=v"(ad[2]) : "s"(sb), "v"(foff[s][0]));
+    asm volatile("v_add_u32 %0, %1, %2" : "=v"(ad[3]) : "s"(sb), "v"(foff[s][1]));
+  };
+  // fragment f, in the order the MFMAs need them: B0, A0 .. A(TM-1), B1 ..
+  auto read_one = [&](const uint32_t (&ad)[4], v8i (&af)[TM], v8i (&bf)[TN], int f) {
+    const bool is_b = f == 0 || f > TM;
+    const int t = f == 0 ? 0 : (f > TM ? f - TM : f - 1);
+    const v4i lo = *reinterpret_cast<lds_v4i_ptr>(ad[is_b ? 2 : 0] + t * (32 * BK));
+    const v4i hi = *reinterpret_cast<lds_v4i_ptr>(ad[is_b ? 3 : 1] + t * (32 * BK));
+    const v8i v = v8i{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+    if (is_b) bf[t] = v;
+    else af[t] = v;
   };
 
   v16f acc[TN][TM];
@@ -227,63 +249,91 @@ __global__ __launch_bounds__(WM *WN * 64) void gemm_nt_kernel(const GemmArgs p) 
 #pragma unroll
       for (int v = 0; v < 16; ++v) acc[tn][tm][v] = 0.0f;
 
-  // MFMAs lo .. hi-1 (of TM*TN) of one 64-byte step
-  auto mma = [&](v8i (&af)[TM], v8i (&bf)[TN], int lo, int hi) {
-#pragma unroll
-    for (int tn = 0; tn < TN; ++tn)
-#pragma unroll
-      for (int tm = 0; tm < TM; ++tm)
-        if (tn * TM + tm >= lo && tn * TM + tm < hi)
-          // D[i = n][j = m]: B rows feed the "A" port, A rows the "B" port
-          acc[tn][tm] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(bf[tn], af[tm], acc[tn][tm], 0, 0, 0, 0, 0, 0);
+  // MFMA number idx (of TM*TN) of one 64-byte step
+  auto mma_one = [&](v8i (&af)[TM], v8i (&bf)[TN], int idx) {
+    const int tn = idx / TM, tm = idx % TM;
+    // D[i = n][j = m]: B rows feed the "A" port, A rows the "B" port
+    acc[tn][tm] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(bf[tn], af[tm], acc[tn][tm], 0, 0, 0, 0, 0, 0);
   };
 
-  // prologue: R units in flight, K tile 0 published, its first half read
+  // The loads of one trip are two units.  The first is spread over the MFMAs of
+  // the first half, the second over those of the second half: a burst of all
+  // of them after the barrier would keep the waves queueing at the
+  // vector-memory port instead of issuing MFMAs.
+  //   prologue: units 0 .. R-2 in flight, K tile 0 published, its first half read
 #pragma unroll
-  for (int u = 0; u < R; ++u) issue_unit(u);
+  for (int u = 0; u < R - 1; ++u) {
+#pragma unroll
+    for (int i = 0; i < ((u & 1) ? IB : IA); ++i) load_one(u & 1, u >> 1, u, i);
+  }
   v8i af0[TM], bf0[TN], af1[TM], bf1[TN];
+  uint32_t ad[4];
   L8_WAIT_VM_LGKM0(PEND0);
   asm volatile("" ::: "memory");
   __builtin_amdgcn_s_barrier();
   asm volatile("" ::: "memory");
-  read_frags(0, 0, af0, bf0);
+  frag_addrs(0, 1, 0, ad);
+#pragma unroll
+  for (int f = 0; f < TM + TN; ++f) read_one(ad, af0, bf0, f);
 
   // One trip = one K tile of 128 = two matrix-core steps of 64.
-  //   first half : MFMAs on (kt, step 0) while (kt, step 1) is read from LDS;
+  //   first half : MFMAs on (kt, step 0) while (kt, step 1) is read from LDS and
+  //                unit 2kt+R-1 is requested (its slot, of K tile kt-1, was
+  //                released at the previous barrier);
   //   barrier    : every wave has now read all of K tile kt (lgkmcnt 0), and
-  //                K tile kt+1 has landed for every wave (partial vmcnt wait),
-  //                so the two slots of K tile kt are refilled with the next
-  //                two units of the sequence;
-  //   second half: MFMAs on (kt, step 1) while (kt+1, step 0) is read.
-  // A wave issues in order, so LDS reads and global loads are spread between
-  // the MFMAs instead of queueing in front of them.
-  constexpr int N_MMA = TM * TN, N_DSR = 2 * (TM + TN);
+  //                K tile kt+1 has landed for every wave (partial vmcnt wait);
+  //   second half: MFMAs on (kt, step 1) while (kt+1, step 0) is read and unit
+  //                2kt+R is requested into the slot K tile kt just released.
+  // Each group below is one MFMA plus its share of the LDS reads and of the
+  // loads; the scheduling fences keep the groups in this order.
+  constexpr int N_MMA = TM * TN, NF = TM + TN;
   constexpr int STRADDLE = L8_STRADDLE < N_MMA - 2 ? L8_STRADDLE : 0;
+  constexpr int S1 = N_MMA - STRADDLE;  // MFMA groups before the barrier
+  constexpr int S2 = N_MMA + STRADDLE;  // and after it
+  constexpr int SR = N_MMA > 2 ? N_MMA - 2 : N_MMA;  // the last two groups of a trip are left without reads
+  constexpr bool U1_IS_B = ((R - 1) & 1) != 0, U2_IS_B = (R & 1) != 0;  // panel kind of units 2kt+R-1 and 2kt+R
+  constexpr int I1 = U1_IS_B ? IB : IA, I2 = U2_IS_B ? IB : IA;
+  int s0 = 0;  // ring slot of unit 2kt
   for (int kt = 0; kt < KT; ++kt) {
-    if (L8_GEMM_DIAG != 2 && L8_GEMM_DIAG != 4) {
-      read_frags(kt, 1, af1, bf1);
-      mma(af0, bf0, 0, N_MMA - STRADDLE);
-      interleave_step<N_MMA - STRADDLE, N_DSR, 0, 0>();
+    const int slot_u1 = wrap(s0 + R - 1);  // unit 2kt+R-1 reuses the slot of unit 2kt-1
+    frag_addrs(s0, wrap(s0 + 1), 1, ad);
+#pragma unroll
+    for (int i = 0; i < S1; ++i) {
+      if (L8_GEMM_DIAG != 2 && L8_GEMM_DIAG != 4) {
+        mma_one(af0, bf0, i);
+#pragma unroll
+        for (int f = (NF * i) / S1; f < (NF * (i + 1)) / S1; ++f) read_one(ad, af1, bf1, f);
+      }
+      if (L8_GEMM_DIAG != 1) {
+#pragma unroll
+        for (int j = (I1 * i) / S1; j < (I1 * (i + 1)) / S1; ++j) load_one(U1_IS_B, kt + (R - 1) / 2, slot_u1, j);
+      }
+      __builtin_amdgcn_sched_barrier(0);
     }
-    __builtin_amdgcn_sched_barrier(0);
     L8_WAIT_VM_LGKM0(PEND);
     asm volatile("" ::: "memory");
     __builtin_amdgcn_s_barrier();
     asm volatile("" ::: "memory");
-    if (L8_GEMM_DIAG != 1) {
-      issue_unit(2 * kt + R);
-      issue_unit(2 * kt + R + 1);
-    }
-    if (L8_GEMM_DIAG != 2 && L8_GEMM_DIAG != 4) {
-      // the last MFMAs of the first half are issued after the barrier: they need
-      // registers only and keep the matrix cores busy while the waves regroup
-      mma(af0, bf0, N_MMA - STRADDLE, N_MMA);
+    // the last MFMAs of the first half are issued after the barrier: they need
+    // registers only and keep the matrix cores busy while the waves regroup
+    frag_addrs(wrap(s0 + 2), wrap(s0 + 3), 0, ad);
+#pragma unroll
+    for (int i = 0; i < S2; ++i) {
+      if (L8_GEMM_DIAG != 2 && L8_GEMM_DIAG != 4) {
+        if (i < STRADDLE) mma_one(af0, bf0, S1 + i);
+        else mma_one(af1, bf1, i - STRADDLE);
+        if (i >= STRADDLE) {  // (kt+1, step 0) replaces the fragments the straddling MFMAs have just consumed
+#pragma unroll
+          for (int f = (NF * (i - STRADDLE)) / SR; f < (NF * (i - STRADDLE + 1)) / SR && f < NF; ++f) read_one(ad, af0, bf0, f);
+        }
+      }
+      if (L8_GEMM_DIAG != 1) {
+#pragma unroll
+        for (int j = (I2 * i) / S2; j < (I2 * (i + 1)) / S2; ++j) load_one(U2_IS_B, kt + R / 2, s0, j);
+      }
       __builtin_amdgcn_sched_barrier(0);
-      read_frags(kt + 1, 0, af0, bf0);
-      mma(af1, bf1, 0, N_MMA);
-      interleave_step<N_MMA, N_DSR, (L8_GEMM_DIAG == 1 ? 0 : NA + NB), 0>();
     }
-    __builtin_amdgcn_sched_barrier(0);
+    s0 = wrap(s0 + 2);
   }
   // drain the tail loads (out of range, zero-filling) before LDS is released
   L8_WAIT_VM_LGKM0(0);
@@ -373,23 +423,28 @@ struct Algo {
   int bm, bn, threads, lds;
 };
 
-// X(WM, WN, TM, TN, R, GROUP_M) -- 1-based position in this list is the `algo` number
-#define L8_ALGO_LIST(X)                                                       \
-  X(2, 4, 4, 2, 5, 4)  /* 1: 256x256, 8 waves (128x64 each), ring of 5     */ \
-  X(2, 4, 4, 2, 4, 4)  /* 2: same, ring of 4 (two whole K tiles)           */ \
-  X(2, 2, 4, 4, 5, 4)  /* 3: 256x256, 4 waves (128x128 each), ring of 5    */ \
-  X(4, 2, 2, 4, 5, 4)  /* 4: 256x256, 8 waves (64x128 each), ring of 5     */ \
-  X(2, 2, 2, 2, 5, 4)  /* 5: 128x128, 4 waves (small problems)             */ \
-  X(2, 4, 4, 2, 5, 8)  /* 6: algo 1 with taller groups                     */ \
-  X(2, 4, 4, 2, 5, 2)  /* 7: algo 1 with shorter groups                    */
+// X(WM, WN, TM, TN, R, GROUP_M, PF) -- 1-based position in this list is the `algo` number
+#define L8_ALGO_LIST(X)                                                          \
+  X(2, 4, 4, 2, 5, 4, 0)  /* 1: 256x256, 8 waves (128x64 each), ring of 5     */ \
+  X(2, 4, 4, 2, 4, 4, 0)  /* 2: same, ring of 4 (two whole K tiles)           */ \
+  X(2, 2, 4, 4, 5, 4, 0)  /* 3: 256x256, 4 waves (128x128 each), ring of 5    */ \
+  X(4, 2, 2, 4, 5, 4, 0)  /* 4: 256x256, 8 waves (64x128 each), ring of 5     */ \
+  X(2, 2, 2, 2, 5, 4, 0)  /* 5: 128x128, 4 waves (small problems)             */ \
+  X(2, 4, 4, 2, 5, 8, 0)  /* 6: algo 1 with taller groups                     */ \
+  X(2, 4, 4, 2, 5, 2, 0)  /* 7: algo 1 with shorter groups                    */ \
+  X(2, 4, 4, 2, 5, 4, 4)  /* 8: algo 1 with L2 touches 4 K tiles ahead        */ \
+  X(2, 4, 4, 2, 5, 4, 8)  /* 9: algo 1 with L2 touches 8 K tiles ahead        */ \
+  X(2, 4, 4, 2, 5, 8, 6)  /* 10: taller groups, touches 6 ahead               */ \
+  X(2, 2, 4, 4, 5, 8, 0)  /* 11: algo 3 with taller groups                    */ \
+  X(2, 2, 4, 4, 5, 4, 4)  /* 12: algo 3 with L2 touches 4 K tiles ahead       */
 
-#define L8_INSTANTIATE(WM, WN, TM, TN, R, GM) \
-  template __global__ void gemm_nt_kernel<WM, WN, TM, TN, R, GM>(const GemmArgs);
+#define L8_INSTANTIATE(WM, WN, TM, TN, R, GM, PF) \
+  template __global__ void gemm_nt_kernel<WM, WN, TM, TN, R, GM, PF>(const GemmArgs);
 L8_ALGO_LIST(L8_INSTANTIATE)
 
 #define L8_MAX2(a, b) ((a) > (b) ? (a) : (b))
-#define L8_ALGO_ROW(WM, WN, TM, TN, R, GM)                                                      \
-  {"mt" #WM "x" #WN "w_" #TM "x" #TN "t_r" #R "_g" #GM, gemm_nt_kernel<WM, WN, TM, TN, R, GM>, \
+#define L8_ALGO_ROW(WM, WN, TM, TN, R, GM, PF)                                                                \
+  {"mt" #WM "x" #WN "w_" #TM "x" #TN "t_r" #R "_g" #GM "_pf" #PF, gemm_nt_kernel<WM, WN, TM, TN, R, GM, PF>, \
    WM * TM * 32, WN * TN * 32, WM * WN * 64, R * L8_MAX2(WM * TM * 32, WN * TN * 32) * 128},
 
 static const Algo kAlgos[] = {L8_ALGO_LIST(L8_ALGO_ROW)};
@@ -409,7 +464,7 @@ static int pick_algo(int64_t M, int64_t N, int64_t K) {
   // large problems: 256x256; problems that would leave most of the chip idle
   // with big tiles: 128x128
   const int64_t big_tiles = ((M + 255) / 256) * ((N + 255) / 256);
-  if (big_tiles >= num_cus()) return 1;
+  if (big_tiles >= num_cus()) return 3;
   return 5;
 }
 
