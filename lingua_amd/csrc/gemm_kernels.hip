@@ -335,23 +335,30 @@ __global__ __launch_bounds__(WM *WN * 64) void gemm_nt_kernel(const GemmArgs p) 
     }
     s0 = wrap(s0 + 2);
   }
-  // drain the tail loads (out of range, zero-filling) before LDS is released
+  // every wave's tail loads (out of range, zero-filling) and LDS reads are done
+  // before the ring is reused as the staging area of the C tile
   L8_WAIT_VM_LGKM0(0);
+  __builtin_amdgcn_s_barrier();
 
   // ---- epilogue ----
   // lane (l31, h) of tile (tn, tm) holds m = l31 and, in accumulator quad qd,
   // n = 8*qd + 4*h + {0..3}.  After the half-wave swap, lanes with h == 0 hold
-  // n = 0..15 and lanes with h == 1 hold n = 16..31 of row m.
+  // n = 0..15 and lanes with h == 1 hold n = 16..31 of row m: 32 bytes of bf16.
+  // Stored from there, every store instruction would scatter 16-byte pieces
+  // over 32 rows.  The tile goes through LDS instead (rows padded by 16 bytes
+  // so that the 16 lanes of a write phase hit 16 different bank groups) and
+  // leaves as whole rows: one store instruction covers 1 KiB of consecutive
+  // bytes of C per row pair.
+  constexpr int C_ROW = BN * 2 + 16;  // staged row pitch in bytes
+  static_assert(BM * C_ROW <= R * UNIT, "the C tile must fit in the ring");
+  typedef __attribute__((address_space(3))) v4i *lds_v4i_wptr;
   const float sa_s = p.sa[0], sb_s = p.sb[0];
   float sav[TM];
-  bool m_okv[TM];
 #pragma unroll
   for (int tm = 0; tm < TM; ++tm) {
     const int m = m0 + (wm * TM + tm) * 32 + l31;
-    m_okv[tm] = m < p.M;
-    sav[tm] = p.sa_row ? (m_okv[tm] ? p.sa[m] : 0.0f) : sa_s;
+    sav[tm] = p.sa_row ? (m < p.M ? p.sa[m] : 0.0f) : sa_s;
   }
-  const bool c_vec = (p.ldc % 8 == 0) && (((uintptr_t)p.C & 15) == 0);
 #pragma unroll
   for (int tn = 0; tn < TN; ++tn) {
     const int nt0 = n0 + (wn * TN + tn) * 32;
@@ -368,7 +375,6 @@ __global__ __launch_bounds__(WM *WN * 64) void gemm_nt_kernel(const GemmArgs p) 
       }
 #pragma unroll
     for (int tm = 0; tm < TM; ++tm) {
-      const int m = m0 + (wm * TM + tm) * 32 + l31;
       const float sa = sav[tm];
       uint32_t pk[8];  // quad qd -> pk[2qd], pk[2qd+1]
 #pragma unroll
@@ -393,18 +399,31 @@ __global__ __launch_bounds__(WM *WN * 64) void gemm_nt_kernel(const GemmArgs p) 
       }
       // lower lanes: pk[0,1]=n0..3 pk[4,5]=n4..7 pk[2,3]=n8..11 pk[6,7]=n12..15
       // upper lanes: pk[0,1]=n16..19 pk[4,5]=n20..23 pk[2,3]=n24..27 pk[6,7]=n28..31
-      const int nbase = nt0 + 16 * h;
-      if (m_okv[tm] && (L8_GEMM_DIAG != 3 || pk[0] == 0x12345678u)) {
-        uint16_t *dst = p.C + (int64_t)m * p.ldc + nbase;
-        if (c_vec && nbase + 16 <= p.N) {
-          *(v4i *)dst = v4i{(int)pk[0], (int)pk[1], (int)pk[4], (int)pk[5]};
-          *(v4i *)(dst + 8) = v4i{(int)pk[2], (int)pk[3], (int)pk[6], (int)pk[7]};
-        } else {
-          const uint32_t all[8] = {pk[0], pk[1], pk[4], pk[5], pk[2], pk[3], pk[6], pk[7]};
+      const uint32_t at = lds0 + ((wm * TM + tm) * 32 + l31) * C_ROW + ((wn * TN + tn) * 32 + 16 * h) * 2;
+      *reinterpret_cast<lds_v4i_wptr>(at) = v4i{(int)pk[0], (int)pk[1], (int)pk[4], (int)pk[5]};
+      *reinterpret_cast<lds_v4i_wptr>(at + 16) = v4i{(int)pk[2], (int)pk[3], (int)pk[6], (int)pk[7]};
+    }
+  }
+  __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0): this wave's part of the tile is in LDS
+  __builtin_amdgcn_s_barrier();
+  // 16-byte chunk c of the tile: row c / CPR, columns 8 * (c % CPR) .. +7
+  constexpr int CPR = BN / 8, CHUNKS = BM * CPR;
+  static_assert(CHUNKS % (NW * 64) == 0, "whole wave stores");
+  const bool c_vec = (p.ldc % 8 == 0) && (((uintptr_t)p.C & 15) == 0);
 #pragma unroll
-          for (int e = 0; e < 16; ++e)
-            if (nbase + e < p.N) dst[e] = (uint16_t)(all[e >> 1] >> (16 * (e & 1)));
-        }
+  for (int it = 0; it < CHUNKS / (NW * 64); ++it) {
+    const int c = (it * NW + wave) * 64 + lane;
+    const int row = c / CPR, col = (c % CPR) * 8;
+    const v4i v = *reinterpret_cast<lds_v4i_ptr>(lds0 + row * C_ROW + col * 2);
+    const int m = m0 + row, n = n0 + col;
+    if (m < p.M && n < p.N && L8_GEMM_DIAG != 3) {
+      uint16_t *dst = p.C + (int64_t)m * p.ldc + n;
+      if (c_vec && n + 8 <= p.N) {
+        *(v4i *)dst = v;
+      } else {
+#pragma unroll
+        for (int e = 0; e < 8; ++e)
+          if (n + e < p.N) dst[e] = (uint16_t)((uint32_t)v[e >> 1] >> (16 * (e & 1)));
       }
     }
   }
@@ -425,18 +444,16 @@ struct Algo {
 
 // X(WM, WN, TM, TN, R, GROUP_M, PF) -- 1-based position in this list is the `algo` number
 #define L8_ALGO_LIST(X)                                                          \
-  X(2, 4, 4, 2, 5, 4, 0)  /* 1: 256x256, 8 waves (128x64 each), ring of 5     */ \
-  X(2, 4, 4, 2, 4, 4, 0)  /* 2: same, ring of 4 (two whole K tiles)           */ \
-  X(2, 2, 4, 4, 5, 4, 0)  /* 3: 256x256, 4 waves (128x128 each), ring of 5    */ \
-  X(4, 2, 2, 4, 5, 4, 0)  /* 4: 256x256, 8 waves (64x128 each), ring of 5     */ \
-  X(2, 2, 2, 2, 5, 4, 0)  /* 5: 128x128, 4 waves (small problems)             */ \
-  X(2, 4, 4, 2, 5, 8, 0)  /* 6: algo 1 with taller groups                     */ \
-  X(2, 4, 4, 2, 5, 2, 0)  /* 7: algo 1 with shorter groups                    */ \
-  X(2, 4, 4, 2, 5, 4, 4)  /* 8: algo 1 with L2 touches 4 K tiles ahead        */ \
-  X(2, 4, 4, 2, 5, 4, 8)  /* 9: algo 1 with L2 touches 8 K tiles ahead        */ \
-  X(2, 4, 4, 2, 5, 8, 6)  /* 10: taller groups, touches 6 ahead               */ \
-  X(2, 2, 4, 4, 5, 8, 0)  /* 11: algo 3 with taller groups                    */ \
-  X(2, 2, 4, 4, 5, 4, 4)  /* 12: algo 3 with L2 touches 4 K tiles ahead       */
+  X(2, 2, 4, 4, 5, 4, 0)  /* 1: 256x256, 4 waves (128x128 each), ring of 5    */ \
+  X(2, 2, 2, 2, 5, 4, 0)  /* 2: 128x128, 4 waves (small problems)             */ \
+  X(2, 4, 4, 2, 5, 4, 0)  /* 3: 256x256, 8 waves (128x64 each)                */ \
+  X(4, 2, 2, 4, 5, 4, 0)  /* 4: 256x256, 8 waves (64x128 each)                */ \
+  X(2, 2, 4, 4, 5, 8, 0)  /* 5: algo 1 with taller groups                     */ \
+  X(2, 2, 4, 4, 5, 2, 0)  /* 6: algo 1 with shorter groups                    */ \
+  X(2, 2, 4, 4, 5, 4, 4)  /* 7: algo 1 with L2 touches 4 K tiles ahead        */ \
+  X(2, 4, 4, 2, 5, 4, 4)  /* 8: algo 3 with L2 touches 4 K tiles ahead        */ \
+  X(2, 2, 4, 4, 5, 16, 0) /* 9: algo 1 with groups of 16                      */ \
+  X(2, 4, 4, 2, 5, 8, 0)  /* 10: algo 3 with taller groups                    */
 
 #define L8_INSTANTIATE(WM, WN, TM, TN, R, GM, PF) \
   template __global__ void gemm_nt_kernel<WM, WN, TM, TN, R, GM, PF>(const GemmArgs);
@@ -460,12 +477,13 @@ extern "C" const char *l8_gemm_algo_name(int algo) {
 }
 
 static int pick_algo(int64_t M, int64_t N, int64_t K) {
-  (void)K;
-  // large problems: 256x256; problems that would leave most of the chip idle
-  // with big tiles: 128x128
+  // large problems: 256x256 tiles -- four waves with 128x128 wave tiles (least
+  // LDS traffic per flop) when the K loop dominates, eight waves when K is short
+  // and the C tile's trip through LDS and out to memory weighs more; problems
+  // that would leave most of the chip idle with big tiles: 128x128
   const int64_t big_tiles = ((M + 255) / 256) * ((N + 255) / 256);
-  if (big_tiles >= num_cus()) return 3;
-  return 5;
+  if (big_tiles >= num_cus()) return K >= 8192 ? 5 : 3;
+  return 2;
 }
 
 extern "C" int l8_gemm_nt(const void *A, const void *B, int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldb,

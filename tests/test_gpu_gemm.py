@@ -42,7 +42,7 @@ def test_exact_small_integer_operands(algo):
         assert torch.equal(out.cpu().double(), want), (algo, M, N, K)
 
 
-@pytest.mark.parametrize("algo", [0, 1, 3, 5])
+@pytest.mark.parametrize("algo", [0, 1, 2, 3])
 def test_k_indexing_with_one_hot_operands(algo):
     # B[n] is one-hot at k = pi(n): C[m,n] = A[m, pi(n)] exactly, for any K (tails included)
     from lingua_amd import ops
