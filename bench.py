@@ -28,7 +28,7 @@ PEAK_FP8_TFLOPS = 5000.0                     # MI355X dense fp8 MFMA, published
 PEAK_HBM_GBPS = 8000.0                       # MI355X HBM3E, published
 # HBM-side bytes per forward-shape GEMM launch from rocprofv3 FETCH_SIZE / WRITE_SIZE, each scaled by what the
 # same counter reads for a 256 MiB copy (profiles/gemm_nt_7b_fwd_hbm_traffic.txt): 1.126 GB read + 0.440 GB written
-GEMM_TRAFFIC_BYTES = 1_566_000_000
+GEMM_TRAFFIC_BYTES = 1_488_000_000
 
 
 def parse():
