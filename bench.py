@@ -38,11 +38,14 @@ def parse():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--algo", type=int, default=0, help="GEMM tile configuration (0 = library default)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--cpu-sample-tokens", type=int, default=2048)
+    ap.add_argument("--cpu-sample-tokens", type=int, default=16384)
     ap.add_argument("--no-kernel-timing", action="store_true", help="do not record per-kernel events in the timed steps")
     ap.add_argument("--workload", choices=["mlp7b", "llama1b"], default="mlp7b",
                     help="mlp7b = the headline workload; llama1b = full Llama-1B-shaped forward+backward step "
                          "(25 layers, dim 2048, ffn 8192, vocab 128256, 4 x 4096 tokens), reported in tokens/s")
+    ap.add_argument("--no-extras", action="store_true",
+                    help="skip the two side measurements: the fused-SwiGLU variant of the same MLP and "
+                         "torch._scaled_mm (what the reference calls) on the step's GEMM shapes")
     ap.add_argument("--kernel-only", choices=["gemm", "copy"], default=None,
                     help="profiling aid: launch only the forward-shape GEMM, or a plain 256 MiB device copy "
                          "(the reference point the FETCH_SIZE / WRITE_SIZE counters are scaled by), a few times")
@@ -97,6 +100,43 @@ def cpu_baseline(torch, sample_tokens):
         "sample": f"same MLP fwd+bwd on {sample_tokens} of {TOKENS} tokens, one repetition, {dt:.2f} s "
                   f"(PyTorch CPU ops: amax/clamp/div/reciprocal/mul/to(float8_e4m3fn), dequantise, fp32 matmul, bf16)",
     }
+
+
+def extras(torch, mlp, timed, args):
+    """Side measurements, never part of `value`:
+    fused_swiglu     the same MLP, same recipe, through lingua_amd.swiglu.Fp8FeedForward (gate fused into the casts,
+                     x quantised once for w1 and w3);
+    torch_scaled_mm  torch._scaled_mm with row-wise scales -- the call the reference makes (lingua/float8.py:65-72) --
+                     on the nine GEMM shapes of one step, same GPU; None where this PyTorch build refuses it."""
+    from lingua_amd.swiglu import Fp8FeedForward
+    res = {}
+    fused = Fp8FeedForward(mlp.w1, mlp.w3, mlp.w2)
+    dt = timed(fused, None)
+    res["fused_swiglu"] = {"value": round(STEP_FLOP / (dt / args.steps) / 1e12, 2), "unit": "TFLOP/s",
+                           "ms_per_step": round(dt / args.steps * 1e3, 4)}
+    try:
+        dev = mlp.w1.weight.device
+        total_ms = 0.0
+        for (M, N, K), count in (((TOKENS, FFN, DIM), 3), ((TOKENS, DIM, FFN), 3), ((FFN, DIM, TOKENS), 3)):
+            a = torch.randn(M, K, device=dev).to(torch.float8_e4m3fn)
+            b = torch.randn(N, K, device=dev).to(torch.float8_e4m3fn)
+            sa = torch.ones(M, 1, device=dev)
+            sb = torch.ones(1, N, device=dev)
+            for _ in range(5):
+                torch._scaled_mm(a, b.t(), scale_a=sa, scale_b=sb, out_dtype=torch.bfloat16)
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            for _ in range(10):
+                torch._scaled_mm(a, b.t(), scale_a=sa, scale_b=sb, out_dtype=torch.bfloat16)
+            e1.record()
+            torch.cuda.synchronize()
+            total_ms += count * e0.elapsed_time(e1) / 10
+        res["torch_scaled_mm"] = {"avg_ms": round(total_ms / 9, 4), "TFLOP/s": round(STEP_FLOP / (total_ms * 1e-3) / 1e12, 1),
+                                  "what": "hipBLASLt through torch._scaled_mm, row-wise scales, mean over the step's 9 GEMMs"}
+    except Exception as exc:  # not every PyTorch build has the row-wise kernel
+        res["torch_scaled_mm"] = None
+        res["torch_scaled_mm_error"] = str(exc)[:200]
+    return res
 
 
 def run_llama1b(args, torch, dev):
@@ -189,26 +229,29 @@ def main():
     x = torch.randn(TOKENS, DIM, generator=g).to(torch.bfloat16).to(dev).requires_grad_(True)
     gy = (torch.randn(TOKENS, DIM, generator=g) * 1e-2).to(torch.bfloat16).to(dev)
 
-    def step():
-        for p in mlp.parameters():
-            p.grad = None
-        x.grad = None
-        y = mlp(x)
-        y.backward(gy)
+    def timed(module, records):
+        def step():
+            for p in module.parameters():
+                p.grad = None
+            x.grad = None
+            y = module(x)
+            y.backward(gy)
 
-    for _ in range(args.warmup):
-        step()
-    torch.cuda.synchronize()
+        for _ in range(args.warmup):
+            step()
+        torch.cuda.synchronize()
+        ops.kernel_timer = records
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(args.steps):
+            step()
+        torch.cuda.synchronize()
+        elapsed = time.perf_counter() - t0
+        ops.kernel_timer = None
+        return elapsed
 
     records = None if args.no_kernel_timing else []
-    ops.kernel_timer = records
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for _ in range(args.steps):
-        step()
-    torch.cuda.synchronize()
-    dt = time.perf_counter() - t0
-    ops.kernel_timer = None
+    dt = timed(mlp, records)
 
     ms_per_step = dt / args.steps * 1e3
     tflops = STEP_FLOP / (dt / args.steps) / 1e12
@@ -257,6 +300,8 @@ def main():
         "roofline": roofline,
         "kernels": kernels,
     }
+    if not args.no_extras:
+        out["extras"] = extras(torch, mlp, timed, args)
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline(torch, args.cpu_sample_tokens)
     print(json.dumps(out))

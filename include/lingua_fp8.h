@@ -105,6 +105,37 @@ int l8_gemm_nt(const void *A, const void *B, int64_t M, int64_t N, int64_t K,
                const float *sa, int sa_mode, const float *sb, int sb_mode,
                const void *bias, void *C, int64_t ldc, int algo, void *stream);
 
+/* SwiGLU gate fused with the row-wise cast of the w2 input.
+ * Replaces `F.silu(self.w1(x)) * self.w3(x)` of lingua/transformer.py:469-471 (two bf16
+ * elementwise kernels) followed by the cast of that product in Fp8LinearFn.forward
+ * (lingua/float8.py:86-87 + :43-47):
+ *   h = bf16( bf16(silu(h1)) * h3 ),  silu(x) = x / (1 + exp(-x)) in fp32,
+ *   then amax / scale / q of h as l8_cast_rowwise.
+ *   h1, h3   bf16 [R,C] (ld1, ld3)
+ *   h        bf16 [R,C] (ldh) or NULL when the caller does not need the product itself
+ *   q, scale, amax, col_amax, workspace: as l8_cast_rowwise; the workspace needs
+ *            l8_swiglu_workspace(R, C) / 2 bytes.
+ * Requires C % 8 == 0, C <= 32768, every leading dimension % 8 == 0. */
+int l8_swiglu_cast_rowwise(const void *h1, const void *h3, int64_t R, int64_t C, int64_t ld1, int64_t ld3,
+                           void *h, int64_t ldh, void *q, int64_t ldq, float *scale, void *amax,
+                           float *col_amax, void *workspace, int64_t workspace_bytes, void *stream);
+int64_t l8_swiglu_workspace(int64_t R, int64_t C);
+
+/* Backward of the SwiGLU gate fused with the row-wise casts of its two gradients.
+ * Replaces autograd's mul / silu_backward kernels for lingua/transformer.py:469-471 and the
+ * casts of grad_out in the backward of w1 and w3 (lingua/float8.py:112-114 + :43-47):
+ *   g3 = bf16( dh * bf16(silu(h1)) )
+ *   g1 = bf16( bf16(dh * h3) * sig * (1 + h1 * (1 - sig)) ),  sig = 1 / (1 + exp(-h1))
+ *   then q1 / scale1 and q3 / scale3 as l8_cast_rowwise of g1 and g3.
+ *   dh, h1, h3 bf16 [R,C];  g1, g3 bf16 [R,C] (ldg) are always written (wgrad needs them);
+ *   col_amax1, col_amax3 fp32 [C]: both or neither; workspace of l8_swiglu_workspace(R, C) bytes with them.
+ * Requires C % 8 == 0, C <= 16384, every leading dimension % 8 == 0. */
+int l8_swiglu_bwd_cast_rowwise(const void *dh, const void *h1, const void *h3, int64_t R, int64_t C,
+                               int64_t lddh, int64_t ld1, int64_t ld3, void *g1, void *g3, int64_t ldg,
+                               void *q1, void *q3, int64_t ldq, float *scale1, float *scale3,
+                               float *col_amax1, float *col_amax3,
+                               void *workspace, int64_t workspace_bytes, void *stream);
+
 int l8_gemm_algo_count(void);
 /* human-readable description of tile configuration `algo` (1-based), or NULL */
 const char *l8_gemm_algo_name(int algo);

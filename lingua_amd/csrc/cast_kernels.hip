@@ -518,7 +518,7 @@ static int64_t rowwise_blocks(int64_t R, int64_t C, bool colmax) {
   return 0;
 }
 
-static int fold_colmax(const void *partials, int64_t slots, int64_t C, float *col_amax, hipStream_t st) {
+int fold_colmax(const void *partials, int64_t slots, int64_t C, float *col_amax, hipStream_t st) {
   hipLaunchKernelGGL(colmax_fold_kernel, dim3((unsigned)((C / 2 + 255) / 256), (unsigned)((slots + 31) / 32)), dim3(256), 0,
                      st, (const uint16_t *)partials, (int)slots, (int)C, (uint32_t *)col_amax);
   L8_HIP(hipGetLastError());

@@ -27,6 +27,10 @@ int fail(int code, const char *fmt, ...);  // records the thread-local message, 
 
 int num_cus();  // compute units of the current device (cached per device)
 
+// Folds partial column maxima [slots, C] (bf16, one row per workgroup of a
+// row-wise kernel) into col_amax[C] (fp32 bit patterns, max-merged).  Defined in cast_kernels.hip.
+int fold_colmax(const void *partials, int64_t slots, int64_t C, float *col_amax, hipStream_t st);
+
 // ---- device side ----------------------------------------------------------
 #define L8_DEV __device__ __forceinline__
 

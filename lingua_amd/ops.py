@@ -182,3 +182,68 @@ def gemm_nt(qa: torch.Tensor, qb: torch.Tensor, sa: torch.Tensor, sb: torch.Tens
 def gemm_algos() -> Tuple[str, ...]:
     lib = _lib.load()
     return tuple(lib.l8_gemm_algo_name(i + 1).decode() for i in range(lib.l8_gemm_algo_count()))
+
+
+def _swiglu_ws(R: int, C: int, device, halves: int):
+    ws_bytes = _lib.load().l8_swiglu_workspace(R, C) // 2 * halves
+    return (torch.empty(ws_bytes, dtype=torch.uint8, device=device) if ws_bytes else None), ws_bytes
+
+
+def swiglu_cast_rowwise(h1: torch.Tensor, h3: torch.Tensor, want_h: bool = True, col_amax: Optional[torch.Tensor] = None):
+    """h = bf16(bf16(silu(h1)) * h3) and its row-wise cast in one pass.
+    Returns (h [R,C] bf16 | None, q [R,C] fp8, scale [R,1] fp32, amax [R,1] bf16); ``col_amax`` as in cast_rowwise."""
+    h1 = _rows_2d(h1, torch.bfloat16, "swiglu_cast_rowwise(h1)")
+    h3 = _rows_2d(h3, torch.bfloat16, "swiglu_cast_rowwise(h3)")
+    if h1.shape != h3.shape or h1.device != h3.device:
+        raise RuntimeError(f"swiglu_cast_rowwise: h1 {tuple(h1.shape)} and h3 {tuple(h3.shape)} must match")
+    st = _prep(h1, "swiglu_cast_rowwise")
+    R, C = h1.shape
+    dev = h1.device
+    h = torch.empty((R, C), dtype=torch.bfloat16, device=dev) if want_h else None
+    q = torch.empty((R, C), dtype=torch.float8_e4m3fn, device=dev)
+    scale = torch.empty((R, 1), dtype=torch.float32, device=dev)
+    amax = torch.empty((R, 1), dtype=torch.bfloat16, device=dev)
+    if col_amax is not None and (col_amax.dtype != torch.float32 or col_amax.numel() != C or not col_amax.is_contiguous()):
+        raise RuntimeError("swiglu_cast_rowwise: col_amax must be a contiguous fp32 tensor with C elements")
+    ws, ws_bytes = _swiglu_ws(R, C, dev, 1) if col_amax is not None else (None, 0)
+    with _timed("swiglu_cast_rowwise", R * C * (5 + (2 if want_h else 0)) + 4 * R, dev):
+        code = _lib.load().l8_swiglu_cast_rowwise(
+            h1.data_ptr(), h3.data_ptr(), R, C, _ld(h1), _ld(h3), h.data_ptr() if want_h else None, C, q.data_ptr(), C,
+            scale.data_ptr(), amax.data_ptr(), col_amax.data_ptr() if col_amax is not None else None,
+            ws.data_ptr() if ws is not None else None, ws_bytes, st)
+    _lib.check(code, "l8_swiglu_cast_rowwise")
+    return h, q, scale, amax
+
+
+def swiglu_bwd_cast_rowwise(dh: torch.Tensor, h1: torch.Tensor, h3: torch.Tensor,
+                            col_amax1: Optional[torch.Tensor] = None, col_amax3: Optional[torch.Tensor] = None):
+    """Gradients of the SwiGLU gate and their row-wise casts in one pass.
+    Returns (g1, g3 [R,C] bf16, q1, q3 [R,C] fp8, scale1, scale3 [R,1] fp32)."""
+    dh = _rows_2d(dh, torch.bfloat16, "swiglu_bwd_cast_rowwise(dh)")
+    h1 = _rows_2d(h1, torch.bfloat16, "swiglu_bwd_cast_rowwise(h1)")
+    h3 = _rows_2d(h3, torch.bfloat16, "swiglu_bwd_cast_rowwise(h3)")
+    if not (dh.shape == h1.shape == h3.shape) or not (dh.device == h1.device == h3.device):
+        raise RuntimeError("swiglu_bwd_cast_rowwise: dh, h1 and h3 must have the same shape and device")
+    if (col_amax1 is None) != (col_amax3 is None):
+        raise RuntimeError("swiglu_bwd_cast_rowwise: pass both column amaxes or neither")
+    st = _prep(dh, "swiglu_bwd_cast_rowwise")
+    R, C = dh.shape
+    dev = dh.device
+    for ca in (col_amax1, col_amax3):
+        if ca is not None and (ca.dtype != torch.float32 or ca.numel() != C or not ca.is_contiguous()):
+            raise RuntimeError("swiglu_bwd_cast_rowwise: column amaxes must be contiguous fp32 tensors with C elements")
+    g1 = torch.empty((R, C), dtype=torch.bfloat16, device=dev)
+    g3 = torch.empty((R, C), dtype=torch.bfloat16, device=dev)
+    q1 = torch.empty((R, C), dtype=torch.float8_e4m3fn, device=dev)
+    q3 = torch.empty((R, C), dtype=torch.float8_e4m3fn, device=dev)
+    s1 = torch.empty((R, 1), dtype=torch.float32, device=dev)
+    s3 = torch.empty((R, 1), dtype=torch.float32, device=dev)
+    ws, ws_bytes = _swiglu_ws(R, C, dev, 2) if col_amax1 is not None else (None, 0)
+    with _timed("swiglu_bwd_cast_rowwise", R * C * 12 + 8 * R, dev):
+        code = _lib.load().l8_swiglu_bwd_cast_rowwise(
+            dh.data_ptr(), h1.data_ptr(), h3.data_ptr(), R, C, _ld(dh), _ld(h1), _ld(h3), g1.data_ptr(), g3.data_ptr(), C,
+            q1.data_ptr(), q3.data_ptr(), C, s1.data_ptr(), s3.data_ptr(),
+            col_amax1.data_ptr() if col_amax1 is not None else None, col_amax3.data_ptr() if col_amax3 is not None else None,
+            ws.data_ptr() if ws is not None else None, ws_bytes, st)
+    _lib.check(code, "l8_swiglu_bwd_cast_rowwise")
+    return g1, g3, q1, q3, s1, s3

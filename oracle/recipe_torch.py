@@ -84,6 +84,21 @@ def linear_fwd_bwd(a, b_t, grad_out, bias=None, wgrad_fp8=True):
     return out, grad_a, grad_b, grad_bias
 
 
+def swiglu_gate(h1: torch.Tensor, h3: torch.Tensor) -> torch.Tensor:
+    """lingua/transformer.py:469-471 between the linears: ``F.silu(h1) * h3`` as eager
+    PyTorch runs it on bf16 tensors (silu in fp32 rounded to bf16, then a bf16 multiply)."""
+    return torch.nn.functional.silu(h1) * h3
+
+
+def swiglu_gate_bwd(dh: torch.Tensor, h1: torch.Tensor, h3: torch.Tensor):
+    """Gradients of ``swiglu_gate`` w.r.t. h1 and h3 as autograd produces them (bf16
+    mul backward twice, silu_backward in fp32 rounded to bf16)."""
+    a = h1.detach().clone().requires_grad_(True)
+    b = h3.detach().clone().requires_grad_(True)
+    swiglu_gate(a, b).backward(dh)
+    return a.grad, b.grad
+
+
 def swiglu_mlp_fwd_bwd(x, w1, w2, w3, grad_y):
     """SwiGLU MLP of lingua/transformer.py:469-471 with every linear in fp8,
     forward and backward; elementwise work in bf16 as eager PyTorch does it."""

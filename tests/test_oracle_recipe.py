@@ -166,3 +166,33 @@ def test_linear_products_c_vs_torch_chain():
 def test_col_sum():
     go = seeded_bf16((50, 24), seed=31)
     assert rel_l2(oracle.col_sum(go), go.float().sum(0)) < 5e-3
+
+
+def test_swiglu_gate_oracle_against_float64_closed_forms():
+    """oracle.recipe_torch.swiglu_gate / swiglu_gate_bwd are the reference's own eager ops; pin them
+    against the closed forms in float64: silu(x) = x / (1 + e^-x), d silu = s (1 + x (1 - s))."""
+    g = torch.Generator().manual_seed(77)
+    h1 = (torch.randn((64, 256), generator=g) * 3).to(torch.bfloat16)
+    h3 = (torch.randn((64, 256), generator=g) * 2).to(torch.bfloat16)
+    dh = (torch.randn((64, 256), generator=g) * 0.1).to(torch.bfloat16)
+    h = rt.swiglu_gate(h1, h3)
+    x, y, d = h1.double(), h3.double(), dh.double()
+    sig = 1.0 / (1.0 + torch.exp(-x))
+    want_h = x * sig * y
+    # two bf16 roundings (silu, product): each at most half an ulp = 2^-8 relative
+    assert h.dtype == torch.bfloat16
+    assert float(((h.double() - want_h).abs() / want_h.abs().clamp_min(1e-30)).max()) <= 2.0 ** -6.95
+    g1, g3 = rt.swiglu_gate_bwd(dh, h1, h3)
+    want_g3 = d * (x * sig)
+    want_g1 = d * y * sig * (1 + x * (1 - sig))
+    assert float(((g3.double() - want_g3).abs() / want_g3.abs().clamp_min(1e-30)).max()) <= 2.0 ** -6.95
+    # the factor 1 + x (1 - s) cancels near x = -1.278: absolute bound scaled by |d y|
+    assert float(((g1.double() - want_g1).abs() / (d * y).abs().clamp_min(1e-30)).max()) <= 1.1 * 2.0 ** -6.95
+    # known answers: silu(0) = 0, silu'(0) = 1/2, silu(40) = 40, silu(-40) = -40 e^-40
+    z = torch.tensor([[0.0, 40.0, -40.0]], dtype=torch.bfloat16)
+    one = torch.ones_like(z)
+    hz = rt.swiglu_gate(z, one).double()[0].tolist()
+    assert hz[0] == 0.0 and hz[1] == 40.0 and abs(hz[2] / (-40.0 * 4.248354255291589e-18) - 1.0) <= 2.0 ** -7.9
+    g1z, g3z = rt.swiglu_gate_bwd(one, z, one)
+    assert g1z[0, :2].tolist() == [0.5, 1.0] and abs(float(g1z[0, 2])) < 1e-14
+    assert g3z[0, :2].tolist() == [0.0, 40.0]
