@@ -15,7 +15,10 @@
 //
 // Every intermediate is rounded to bf16 where the unfused PyTorch chain
 // materialises a bf16 tensor, so the results agree with that chain up to the
-// last bit of the fp32 exp / division.  One 256-thread workgroup per row (wave
+// last bits of the fp32 sigmoid: at most two bf16 ulps apart, identical for
+// more than 99.5 % of the elements (the bound the tests state); amax, scale
+// and e4m3 bytes are then exact functions of the bf16 values produced here.
+// One 256-thread workgroup per row (wave
 // w owns the 512-column chunks w, w+4, ...), the layout of the long-row kernel
 // of cast_kernels.hip; the amax -> scale -> cast stage is shared with it.
 #include "l8_common.h"
@@ -31,8 +34,17 @@ L8_DEV uint32_t bf16_rne_bits(float v) {
 }
 L8_DEV float bf16_round(float v) { return bf16_bits_to_f32(bf16_rne_bits(v)); }
 
-// silu in the form of ATen's kernel: x / (1 + exp(-x)), fp32
-L8_DEV float silu_f32(float x) { return x / (1.0f + expf(-x)); }
+// 1 / (1 + exp(-x)) with the hardware exp2 and reciprocal (about 1 ulp of fp32
+// each).  The library exp and the IEEE division cost ~5x the instructions and
+// made these kernels VALU-bound (302 us forward / 550 us backward on
+// [16384, 11008] against ~230 / ~400 us of memory time); every result is
+// rounded to bf16 right away, where an fp32 ulp decides one rounding in ~10^4.
+L8_DEV float sigmoid_f32(float x) {
+  const float e = __builtin_amdgcn_exp2f(x * -1.4426950408889634f);
+  return __builtin_amdgcn_rcpf(1.0f + e);
+}
+// silu(x) = x / (1 + exp(-x)), fp32
+L8_DEV float silu_f32(float x) { return x * sigmoid_f32(x); }
 
 // one element of the forward gate
 L8_DEV uint32_t gate_fwd(float a, float b) { return bf16_rne_bits(bf16_round(silu_f32(a)) * b); }
@@ -46,9 +58,8 @@ L8_DEV uint32_t gate_fwd2(uint32_t a, uint32_t b) {
 
 // one element of the backward gate: d = dh, a = h1, b = h3
 L8_DEV void gate_bwd(float d, float a, float b, uint32_t &g1, uint32_t &g3) {
-  const float e = expf(-a);
-  const float s = bf16_round(a / (1.0f + e));   // what forward saved: bf16 silu(h1)
-  const float sig = 1.0f / (1.0f + e);
+  const float sig = sigmoid_f32(a);
+  const float s = bf16_round(a * sig);          // what forward saved: bf16 silu(h1)
   const float gs = bf16_round(d * b);           // gradient of the silu output, a bf16 tensor in the unfused chain
   g3 = bf16_rne_bits(d * s);
   g1 = bf16_rne_bits((gs * sig) * (1.0f + a * (1.0f - sig)));
