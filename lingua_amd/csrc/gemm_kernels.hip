@@ -335,12 +335,39 @@ __global__ __launch_bounds__(WM *WN * 64) void gemm_nt_kernel(const GemmArgs p) 
     }
     s0 = wrap(s0 + 2);
   }
+  // ---- epilogue ----
+  // All scales of this wave's part of the tile are requested in one batch,
+  // before the wait that drains the ring: one memory latency in total,
+  // overlapped with that wait, instead of one per 32-column tile.
+  const float sa_s = p.sa[0], sb_s = p.sb[0];
+  float sav[TM];
+#pragma unroll
+  for (int tm = 0; tm < TM; ++tm) {
+    const int m = m0 + (wm * TM + tm) * 32 + l31;
+    sav[tm] = p.sa_row ? (m < p.M ? p.sa[m] : 0.0f) : sa_s;
+  }
+  // scales of the 16 n per 32-column tile that this lane holds before the half-wave swap
+  float sbv[TN][4][4];
+  const bool sb_vec = p.sb_row && (((uintptr_t)p.sb & 15) == 0);
+#pragma unroll
+  for (int tn = 0; tn < TN; ++tn)
+#pragma unroll
+    for (int qd = 0; qd < 4; ++qd) {
+      const int nq = n0 + (wn * TN + tn) * 32 + 8 * qd + 4 * h;  // four consecutive n
+      if (sb_vec && nq + 4 <= p.N) {
+        const v4f t = *(const v4f *)(p.sb + nq);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) sbv[tn][qd][e] = t[e];
+      } else {
+#pragma unroll
+        for (int e = 0; e < 4; ++e) sbv[tn][qd][e] = p.sb_row ? (nq + e < p.N ? p.sb[nq + e] : 0.0f) : sb_s;
+      }
+    }
   // every wave's tail loads (out of range, zero-filling) and LDS reads are done
   // before the ring is reused as the staging area of the C tile
   L8_WAIT_VM_LGKM0(0);
   __builtin_amdgcn_s_barrier();
 
-  // ---- epilogue ----
   // lane (l31, h) of tile (tn, tm) holds m = l31 and, in accumulator quad qd,
   // n = 8*qd + 4*h + {0..3}.  After the half-wave swap, lanes with h == 0 hold
   // n = 0..15 and lanes with h == 1 hold n = 16..31 of row m: 32 bytes of bf16.
@@ -352,27 +379,19 @@ __global__ __launch_bounds__(WM *WN * 64) void gemm_nt_kernel(const GemmArgs p) 
   constexpr int C_ROW = BN * 2 + 16;  // staged row pitch in bytes
   static_assert(BM * C_ROW <= R * UNIT, "the C tile must fit in the ring");
   typedef __attribute__((address_space(3))) v4i *lds_v4i_wptr;
-  const float sa_s = p.sa[0], sb_s = p.sb[0];
-  float sav[TM];
-#pragma unroll
-  for (int tm = 0; tm < TM; ++tm) {
-    const int m = m0 + (wm * TM + tm) * 32 + l31;
-    sav[tm] = p.sa_row ? (m < p.M ? p.sa[m] : 0.0f) : sa_s;
-  }
 #pragma unroll
   for (int tn = 0; tn < TN; ++tn) {
-    const int nt0 = n0 + (wn * TN + tn) * 32;
-    // scales and bias of the 16 n this lane holds before the swap
-    float sbv[4][4], biasv[4][4];
+    // the bias (rare: the linears of the model have none) is fetched per 32-column tile
+    float biasv[4][4];
+    if (p.bias) {
 #pragma unroll
-    for (int qd = 0; qd < 4; ++qd)
+      for (int qd = 0; qd < 4; ++qd)
 #pragma unroll
-      for (int e = 0; e < 4; ++e) {
-        const int n = nt0 + 8 * qd + 4 * h + e;
-        const bool n_ok = n < p.N;
-        sbv[qd][e] = p.sb_row ? (n_ok ? p.sb[n] : 0.0f) : sb_s;
-        biasv[qd][e] = (p.bias && n_ok) ? bf16_bits_to_f32(p.bias[n]) : 0.0f;
-      }
+        for (int e = 0; e < 4; ++e) {
+          const int n = n0 + (wn * TN + tn) * 32 + 8 * qd + 4 * h + e;
+          biasv[qd][e] = n < p.N ? bf16_bits_to_f32(p.bias[n]) : 0.0f;
+        }
+    }
 #pragma unroll
     for (int tm = 0; tm < TM; ++tm) {
       const float sa = sav[tm];
@@ -381,7 +400,10 @@ __global__ __launch_bounds__(WM *WN * 64) void gemm_nt_kernel(const GemmArgs p) 
       for (int qd = 0; qd < 4; ++qd) {
         float v[4];
 #pragma unroll
-        for (int e = 0; e < 4; ++e) v[e] = acc[tn][tm][qd * 4 + e] * sa * sbv[qd][e] + biasv[qd][e];
+        for (int e = 0; e < 4; ++e) {
+          v[e] = acc[tn][tm][qd * 4 + e] * sa * sbv[tn][qd][e];
+          if (p.bias) v[e] += biasv[qd][e];
+        }
         typedef __bf16 bf2 __attribute__((ext_vector_type(2)));
         bf2 lo = {(__bf16)v[0], (__bf16)v[1]}, hi = {(__bf16)v[2], (__bf16)v[3]};
         pk[2 * qd] = __builtin_bit_cast(uint32_t, lo);
