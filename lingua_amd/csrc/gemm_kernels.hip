@@ -46,6 +46,8 @@
 // of the main loop to attribute stalls: 1 = no global loads after the prologue,
 // 2 = no LDS reads / matrix-core work, 3 = no stores of C, 4 = as 2 with every workgroup loading the same tile (all
 // L2 hits).  Results are wrong by construction.
+#include <type_traits>
+
 #include "l8_common.h"
 
 namespace l8 {
@@ -379,11 +381,13 @@ __global__ __launch_bounds__(WM *WN * 64) void gemm_nt_kernel(const GemmArgs p) 
   constexpr int C_ROW = BN * 2 + 16;  // staged row pitch in bytes
   static_assert(BM * C_ROW <= R * UNIT, "the C tile must fit in the ring");
   typedef __attribute__((address_space(3))) v4i *lds_v4i_wptr;
+  auto convert_and_stage = [&](auto has_bias) {
+    constexpr bool HAS_BIAS = decltype(has_bias)::value;
 #pragma unroll
   for (int tn = 0; tn < TN; ++tn) {
     // the bias (rare: the linears of the model have none) is fetched per 32-column tile
     float biasv[4][4];
-    if (p.bias) {
+    if constexpr (HAS_BIAS) {
 #pragma unroll
       for (int qd = 0; qd < 4; ++qd)
 #pragma unroll
@@ -402,7 +406,7 @@ __global__ __launch_bounds__(WM *WN * 64) void gemm_nt_kernel(const GemmArgs p) 
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
           v[e] = acc[tn][tm][qd * 4 + e] * sa * sbv[tn][qd][e];
-          if (p.bias) v[e] += biasv[qd][e];
+          if constexpr (HAS_BIAS) v[e] += biasv[qd][e];
         }
         typedef __bf16 bf2 __attribute__((ext_vector_type(2)));
         bf2 lo = {(__bf16)v[0], (__bf16)v[1]}, hi = {(__bf16)v[2], (__bf16)v[3]};
@@ -426,26 +430,40 @@ __global__ __launch_bounds__(WM *WN * 64) void gemm_nt_kernel(const GemmArgs p) 
       *reinterpret_cast<lds_v4i_wptr>(at + 16) = v4i{(int)pk[2], (int)pk[3], (int)pk[6], (int)pk[7]};
     }
   }
+  };
+  if (p.bias) convert_and_stage(std::true_type{});
+  else convert_and_stage(std::false_type{});
   __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0): this wave's part of the tile is in LDS
   __builtin_amdgcn_s_barrier();
   // 16-byte chunk c of the tile: row c / CPR, columns 8 * (c % CPR) .. +7
   constexpr int CPR = BN / 8, CHUNKS = BM * CPR;
   static_assert(CHUNKS % (NW * 64) == 0, "whole wave stores");
   const bool c_vec = (p.ldc % 8 == 0) && (((uintptr_t)p.C & 15) == 0);
+  constexpr int ITERS = CHUNKS / (NW * 64), ROWS_PER_IT = NW * 64 / CPR;
+  static_assert((NW * 64) % CPR == 0, "a wave store covers whole rows");
+  const int row0 = (wave * 64 + lane) / CPR, col = ((wave * 64 + lane) % CPR) * 8;
+  if (c_vec && m0 + BM <= p.M && n0 + BN <= p.N && L8_GEMM_DIAG != 3) {
+    // interior tile: no masks, one pointer and one LDS address stepped by constants
+    uint16_t *dst = p.C + (int64_t)(m0 + row0) * p.ldc + n0 + col;
+    const uint32_t at = lds0 + row0 * C_ROW + col * 2;
 #pragma unroll
-  for (int it = 0; it < CHUNKS / (NW * 64); ++it) {
-    const int c = (it * NW + wave) * 64 + lane;
-    const int row = c / CPR, col = (c % CPR) * 8;
-    const v4i v = *reinterpret_cast<lds_v4i_ptr>(lds0 + row * C_ROW + col * 2);
-    const int m = m0 + row, n = n0 + col;
-    if (m < p.M && n < p.N && L8_GEMM_DIAG != 3) {
-      uint16_t *dst = p.C + (int64_t)m * p.ldc + n;
-      if (c_vec && n + 8 <= p.N) {
-        *(v4i *)dst = v;
-      } else {
+    for (int it = 0; it < ITERS; ++it)
+      *(v4i *)(dst + (int64_t)it * ROWS_PER_IT * p.ldc) = *reinterpret_cast<lds_v4i_ptr>(at + it * (ROWS_PER_IT * C_ROW));
+  } else if (L8_GEMM_DIAG != 3) {
+#pragma unroll 4
+    for (int it = 0; it < ITERS; ++it) {
+      const int row = row0 + it * ROWS_PER_IT;
+      const v4i v = *reinterpret_cast<lds_v4i_ptr>(lds0 + row * C_ROW + col * 2);
+      const int m = m0 + row, n = n0 + col;
+      if (m < p.M && n < p.N) {
+        uint16_t *dst = p.C + (int64_t)m * p.ldc + n;
+        if (c_vec && n + 8 <= p.N) {
+          *(v4i *)dst = v;
+        } else {
 #pragma unroll
-        for (int e = 0; e < 8; ++e)
-          if (n + e < p.N) dst[e] = (uint16_t)((uint32_t)v[e >> 1] >> (16 * (e & 1)));
+          for (int e = 0; e < 8; ++e)
+            if (n + e < p.N) dst[e] = (uint16_t)((uint32_t)v[e >> 1] >> (16 * (e & 1)));
+        }
       }
     }
   }
