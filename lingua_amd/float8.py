@@ -24,6 +24,10 @@ Differences, all deliberate:
   * the Inductor / CUDA-graph side effects of the converter
     (lingua/float8.py:162,187-189) have no counterpart: nothing here is traced
     or compiled at run time;
+  * linears applied to the same activation one after the other (w1 / w3, wq /
+    wk / wv) share its quantised copy within one forward and one backward
+    (``config.share_input_casts``); the reference quantises it once per
+    linear.  Same bytes, fewer passes over the activation;
   * the reference's autograd work-around ``b_t + grad_out[:1,:,None]*0``
     (lingua/float8.py:108) is a no-op for finite gradients and is not issued.
 """
@@ -45,6 +49,10 @@ class Fp8Config:
     fp8_wgrad: bool = True
     # GEMM tile configuration handed to l8_gemm_nt (0 = library default)
     gemm_algo: int = 0
+    # linears that are applied to the very same activation one after the other
+    # (w1 / w3 of the MLP, wq / wk / wv of attention) quantise it once per
+    # forward and once per backward instead of once each
+    share_input_casts: bool = True
 
 
 config = Fp8Config()
@@ -79,6 +87,39 @@ def matmul(first, amax_first, second_t, amax_second_t, bias, use_fast_accum: boo
     return ops.gemm_nt(q1, q2, s1, s2, bias, algo=config.gemm_algo)
 
 
+class _LastCast:
+    """One-entry memo of the last activation quantised.  A lookup hits when it sees the same
+    memory (pointer, shape, strides, dtype, stream) at the same version counter AND comes from
+    a consumer (weight) that has not used the entry yet: the same weight asking again means a
+    new pass over the model, which quantises afresh.  The entry keeps the tensor alive, so its
+    address cannot be handed to another tensor while it is cached; the forward entry is dropped
+    by the first backward that runs and the backward entry by the next forward."""
+
+    def __init__(self):
+        self.key, self.keep, self.value, self.users = None, None, None, set()
+
+    @staticmethod
+    def _key(t):
+        return (t.data_ptr(), tuple(t.shape), tuple(t.stride()), t.dtype, t.device, t._version,
+                torch.cuda.current_stream(t.device).cuda_stream)
+
+    def get(self, t, user):
+        if self.key is None or user in self.users or self.key != self._key(t):
+            return None
+        self.users.add(user)
+        return self.value
+
+    def put(self, t, value, user):
+        self.key, self.keep, self.value, self.users = self._key(t), t, value, {user}
+
+    def clear(self):
+        self.key, self.keep, self.value, self.users = None, None, None, set()
+
+
+_fwd_cast = _LastCast()   # a -> (qa, sa, a_col_amax | None)
+_bwd_cast = _LastCast()   # a -> (qat, sat)
+
+
 class Fp8LinearFn(torch.autograd.Function):
     """``out = a @ b_t.T + bias`` with fp8 operands (lingua/float8.py:83-131)."""
 
@@ -88,8 +129,17 @@ class Fp8LinearFn(torch.autograd.Function):
             raise RuntimeError(f"Fp8LinearFn: bf16 input and weight required, got {a.dtype} and {b_t.dtype}")
         need_wgrad_stats = config.fp8_wgrad and b_t.requires_grad
         # column amaxes of `a` fall out of the row-wise pass; wgrad wants them
-        a_col_amax = torch.zeros(a.shape[1], dtype=torch.float32, device=a.device) if need_wgrad_stats else None
-        qa, sa, _ = ops.cast_rowwise(a, col_amax=a_col_amax)
+        _bwd_cast.clear()
+        hit = _fwd_cast.get(a, b_t.data_ptr()) if config.share_input_casts else None
+        if hit is not None and (hit[2] is not None or not need_wgrad_stats):
+            qa, sa, a_col_amax = hit
+            if not need_wgrad_stats:
+                a_col_amax = None
+        else:
+            a_col_amax = torch.zeros(a.shape[1], dtype=torch.float32, device=a.device) if need_wgrad_stats else None
+            qa, sa, _ = ops.cast_rowwise(a, col_amax=a_col_amax)
+            if config.share_input_casts:
+                _fwd_cast.put(a, (qa, sa, a_col_amax), b_t.data_ptr())
         qb, sb, amax_b_t = ops.cast_rowwise(b_t)
         out = ops.gemm_nt(qa, qb, sa, sb, bias, algo=config.gemm_algo)
 
@@ -115,6 +165,7 @@ class Fp8LinearFn(torch.autograd.Function):
         if grad_out.dtype != torch.bfloat16:
             raise RuntimeError(f"Fp8LinearFn.backward: bf16 grad_out required, got {grad_out.dtype}")
         fp8_wgrad = ctx.fp8_wgrad and ctx.b_requires_grad
+        _fwd_cast.clear()
 
         qg = sg = None
         g_col_amax = None
@@ -133,10 +184,16 @@ class Fp8LinearFn(torch.autograd.Function):
             if fp8_wgrad:
                 if g_col_amax is None:
                     g_col_amax = ops.col_amax(grad_out)
-                if a_col_amax is None:
-                    a_col_amax = ops.col_amax(a)
                 qgt, sgt = ops.cast_colwise_transposed(grad_out, g_col_amax)
-                qat, sat = ops.cast_colwise_transposed(a, a_col_amax)
+                hit = _bwd_cast.get(a, b_t.data_ptr()) if config.share_input_casts else None
+                if hit is not None:
+                    qat, sat = hit
+                else:
+                    if a_col_amax is None:
+                        a_col_amax = ops.col_amax(a)
+                    qat, sat = ops.cast_colwise_transposed(a, a_col_amax)
+                    if config.share_input_casts:
+                        _bwd_cast.put(a, (qat, sat), b_t.data_ptr())
                 grad_b = ops.gemm_nt(qgt, qat, sgt, sat, None, algo=ctx.gemm_algo)
             else:
                 grad_b = grad_out.t() @ a

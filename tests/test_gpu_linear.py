@@ -248,3 +248,50 @@ def test_config5_llama_1b_training_step():
         want = oracle.gemm_nt(qg, qa, sg, sa)
         assert rel_l2(lin.weight.grad[n_idx][:, k_idx], want) <= TOL, name
     assert all(p.grad is not None and torch.isfinite(p.grad.float()).all() for p in model.parameters())
+
+
+def test_linears_on_the_same_activation_share_its_casts():
+    """w1 / w3 style: the second linear on the same input reuses the quantised copy (forward and
+    backward); a new pass quantises afresh; results are bit-identical with sharing off."""
+    from lingua_amd import Fp8Linear, float8, ops
+    torch.manual_seed(5)
+    l1 = Fp8Linear(256, 512, bias=False, device="cuda", dtype=torch.bfloat16)
+    l3 = Fp8Linear(256, 512, bias=False, device="cuda", dtype=torch.bfloat16)
+    x = seeded_bf16((2, 40, 256), seed=21).cuda().requires_grad_(True)
+    g = seeded_bf16((2, 40, 512), std=0.02, seed=22).cuda()
+
+    def run(share):
+        old = float8.config.share_input_casts
+        float8.config.share_input_casts = share
+        rec = []
+        ops.kernel_timer = rec
+        try:
+            for p in (l1.weight, l3.weight, x):
+                p.grad = None
+            y1, y3 = l1(x), l3(x)
+            n_fwd = sum(1 for r in rec if r[0] == "cast_rowwise")
+            (y1 * 2 + y3).backward(g)
+            n_bwd_t = sum(1 for r in rec if r[0] == "cast_colwise_t")
+            # a second forward over the same tensor is a new pass: the activation is quantised again
+            del rec[:]
+            with torch.no_grad():
+                l1(x), l3(x)
+            n_again = sum(1 for r in rec if r[0] == "cast_rowwise")
+        finally:
+            ops.kernel_timer = None
+            float8.config.share_input_casts = old
+        return (y1.detach(), y3.detach(), x.grad.clone(), l1.weight.grad.clone(), l3.weight.grad.clone()), (n_fwd, n_bwd_t, n_again)
+
+    shared, counts_shared = run(True)
+    apart, counts_apart = run(False)
+    assert counts_apart == (4, 4, 4), counts_apart     # x twice + two weights; two grads + x twice
+    assert counts_shared == (3, 3, 3), counts_shared   # x once per pass
+    for a, b in zip(shared, apart):
+        assert torch.equal(a.view(torch.int16), b.view(torch.int16))
+    # an in-place change of the activation is seen (version counter)
+    with torch.no_grad():
+        ya = l1(x)
+        x.mul_(2.0)
+        yb = l3(x)
+        yc = l3(x / 1.0)
+    assert torch.equal(yb, yc) and not torch.equal(ya, yb)
