@@ -46,9 +46,10 @@ def parse():
     ap.add_argument("--no-extras", action="store_true",
                     help="skip the two side measurements: the fused-SwiGLU variant of the same MLP and "
                          "torch._scaled_mm (what the reference calls) on the step's GEMM shapes")
-    ap.add_argument("--kernel-only", choices=["gemm", "copy"], default=None,
+    ap.add_argument("--kernel-only", choices=["gemm", "copy", "casts"], default=None,
                     help="profiling aid: launch only the forward-shape GEMM, or a plain 256 MiB device copy "
-                         "(the reference point the FETCH_SIZE / WRITE_SIZE counters are scaled by), a few times")
+                         "(the reference point the FETCH_SIZE / WRITE_SIZE counters are scaled by), or each cast "
+                         "kernel on its 7B-MLP shape, a few times")
     return ap.parse_args()
 
 
@@ -216,6 +217,39 @@ def main():
         torch.cuda.synchronize()
         print(json.dumps({"kernel_only": "gemm", "M": TOKENS, "N": FFN, "K": DIM, "launches": 3,
                           "algorithmic_bytes": TOKENS * DIM + FFN * DIM + 2 * TOKENS * FFN + 4 * (TOKENS + FFN)}))
+        return
+
+    if args.kernel_only == "casts":
+        g = torch.Generator().manual_seed(3)
+        x = torch.randn(TOKENS, DIM, generator=g).to(torch.bfloat16).to(dev)
+        h1 = torch.randn(TOKENS, FFN, generator=g).to(torch.bfloat16).to(dev)
+        h3 = torch.randn(TOKENS, FFN, generator=g).to(torch.bfloat16).to(dev)
+        w = (torch.randn(FFN, DIM, generator=g) * 0.02).to(torch.bfloat16).to(dev)
+        amax_w = ops.amax_reduce(ops.cast_rowwise(w, want_q=False)[2])
+        col_x = ops.col_amax(x)
+        col_h = ops.col_amax(h1)
+        torch.cuda.synchronize()
+        for _ in range(3):
+            ops.cast_rowwise(x, col_amax=torch.zeros(DIM, dtype=torch.float32, device=dev))
+            ops.cast_rowwise(h1, col_amax=torch.zeros(FFN, dtype=torch.float32, device=dev))
+            ops.cast_rowwise(w)
+            ops.cast_colwise_transposed(x, col_x)
+            ops.cast_colwise_transposed(h1, col_h)
+            ops.cast_tensorwise(w, amax_w, transpose=True)
+            ops.swiglu_cast_rowwise(h1, h3, want_h=True, col_amax=torch.zeros(FFN, dtype=torch.float32, device=dev))
+            ops.swiglu_bwd_cast_rowwise(h1, h3, h1, torch.zeros(FFN, dtype=torch.float32, device=dev),
+                                        torch.zeros(FFN, dtype=torch.float32, device=dev))
+        torch.cuda.synchronize()
+        e = TOKENS * FFN
+        print(json.dumps({"kernel_only": "casts", "launches_each": 3, "compulsory_bytes": {
+            "cast_rowwise x[16384,4096] + col amax": TOKENS * DIM * 3 + 4 * TOKENS + 4 * DIM,
+            "cast_rowwise h[16384,11008] + col amax": e * 3 + 4 * TOKENS + 4 * FFN,
+            "cast_rowwise w[11008,4096]": FFN * DIM * 3 + 4 * FFN,
+            "cast_colwise_transposed x": TOKENS * DIM * 3 + 4 * DIM,
+            "cast_colwise_transposed h": e * 3 + 4 * FFN,
+            "cast_tensorwise transposed w": FFN * DIM * 3 + 4,
+            "swiglu_cast_rowwise (h written)": e * 7 + 4 * TOKENS + 4 * FFN,
+            "swiglu_bwd_cast_rowwise": e * 12 + 8 * TOKENS + 8 * FFN}}))
         return
 
     if args.workload == "llama1b":
