@@ -153,19 +153,28 @@ def run_llama1b(args, torch, dev):
     tokens = torch.randint(0, LLAMA_1B["vocab"], (B, S), generator=g).to(dev)
     labels = torch.randint(0, LLAMA_1B["vocab"], (B, S), generator=g).to(dev)
 
-    def step():
-        for p in model.parameters():
-            p.grad = None
-        model(tokens, labels).backward()
+    def timed(m):
+        def step():
+            for p in m.parameters():
+                p.grad = None
+            m(tokens, labels).backward()
 
-    for _ in range(args.warmup):
-        step()
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for _ in range(args.steps):
-        step()
-    torch.cuda.synchronize()
-    dt = (time.perf_counter() - t0) / args.steps
+        for _ in range(args.warmup):
+            step()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(args.steps):
+            step()
+        torch.cuda.synchronize()
+        return (time.perf_counter() - t0) / args.steps
+
+    dt = timed(model)
+    fused_dt = None
+    if not args.no_extras:
+        # same weights, gate fused into the casts and norms that hand their output over quantised
+        from lingua_amd.norm import fuse_rmsnorm
+        from lingua_amd.swiglu import fuse_feed_forward
+        fused_dt = timed(fuse_rmsnorm(fuse_feed_forward(model)))
     fpt = llama_flops_per_token(LLAMA_1B["n_layers"], LLAMA_1B["dim"], LLAMA_1B["ffn_dim"], LLAMA_1B["vocab"], S)
     fp8_flop = 25 * 3 * (4 * 2 * B * S * 2048 * 2048 + 3 * 2 * B * S * 2048 * 8192)
     print(json.dumps({
@@ -175,6 +184,8 @@ def run_llama1b(args, torch, dev):
         "config": {"workload": "llama-1B step fwd+bwd (configs[4])", "batch": B, "seq_len": S, **LLAMA_1B},
         "model_TFLOP/s": round(fpt * B * S / dt / 1e12, 1),
         "fp8_linear_TFLOP/s_if_alone": round(fp8_flop / dt / 1e12, 1),
+        "extras": None if fused_dt is None else {"fused_swiglu_and_rmsnorm": {
+            "value": round(B * S / fused_dt, 1), "unit": "tokens/s", "ms_per_step": round(fused_dt * 1e3, 3)}},
     }))
 
 

@@ -136,6 +136,21 @@ int l8_swiglu_bwd_cast_rowwise(const void *dh, const void *h1, const void *h3, i
                                float *col_amax1, float *col_amax3,
                                void *workspace, int64_t workspace_bytes, void *stream);
 
+/* RMSNorm fused with the row-wise cast of its output.
+ * Replaces RMSNorm.forward of lingua/transformer.py:283-289 (x.float(), x*x, mean, rsqrt, two
+ * multiplies, type_as: seven eager kernels) followed by the cast of that output in the forward of
+ * the linears it feeds (wq/wk/wv, w1/w3; lingua/float8.py:86-87 + :43-47):
+ *   r = rsqrt(mean(f32(x)^2) + eps);  y = bf16((f32(x) * r) * f32(w));  q, scale = row-wise cast of y.
+ *   x     bf16 [R,C] (ldx);  w [C], bf16 (w_is_f32 == 0) or fp32
+ *   y     bf16 [R,C] (ldy), always written
+ *   q, scale: as l8_cast_rowwise, both or neither;  rstd fp32 [R] = r (may be NULL; what backward needs)
+ *   col_amax, workspace: as l8_cast_rowwise, workspace of l8_rmsnorm_workspace(R, C) bytes
+ * Requires C % 8 == 0, C <= 8192, every leading dimension % 8 == 0. */
+int l8_rmsnorm_cast_rowwise(const void *x, const void *w, int w_is_f32, int64_t R, int64_t C, int64_t ldx,
+                            float eps, void *y, int64_t ldy, void *q, int64_t ldq, float *scale, float *rstd,
+                            float *col_amax, void *workspace, int64_t workspace_bytes, void *stream);
+int64_t l8_rmsnorm_workspace(int64_t R, int64_t C);
+
 int l8_gemm_algo_count(void);
 /* human-readable description of tile configuration `algo` (1-based), or NULL */
 const char *l8_gemm_algo_name(int algo);

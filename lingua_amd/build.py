@@ -10,7 +10,7 @@ import sys
 _HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(_HERE, "csrc")
 LIB_PATH = os.path.join(_HERE, "liblingua_fp8.so")
-SOURCES = ["api.cpp", "cast_kernels.hip", "gemm_kernels.hip", "swiglu_kernels.hip"]
+SOURCES = ["api.cpp", "cast_kernels.hip", "gemm_kernels.hip", "swiglu_kernels.hip", "norm_kernels.hip"]
 
 HIPCC_FLAGS = [
     "--offload-arch=gfx950",

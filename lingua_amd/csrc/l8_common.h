@@ -133,4 +133,33 @@ L8_DEV uint32_t wave_max_u32(uint32_t v) {
   return max(max(a, b), max(c, d));
 }
 
+// fp32 -> bf16 bits, round to nearest even (what a PyTorch op leaves when its fp32 result lands in a bf16 tensor)
+L8_DEV uint32_t bf16_rne_bits(float v) {
+  const __bf16 b = (__bf16)v;
+  return (uint32_t) __builtin_bit_cast(unsigned short, b);
+}
+L8_DEV float bf16_round(float v) { return bf16_bits_to_f32(bf16_rne_bits(v)); }
+
+// amax bits (uniform) -> scale, 1/scale, finite flag, as in the row-wise cast
+struct RowScale {
+  float s, recip;
+  bool finite;
+};
+L8_DEV RowScale row_scale(uint32_t amax_bits) {
+  RowScale r;
+  r.finite = amax_bits < 0x7f80u;
+  r.s = r.finite ? scale_from_amax(bf16_bits_to_f32(amax_bits))
+                 : __uint_as_float(amax_bits == 0x7f80u ? 0x7f800000u : 0x7fc00000u);
+  r.recip = recip_exact(r.s);
+  return r;
+}
+
+// Workgroup-per-row kernels that produce their row on the fly (fused gate, fused
+// norm) keep column maxima in registers (packed pairs, NCHW * 4 dwords per
+// tensor) while that fits the 256-register budget of two workgroups per CU,
+// else in a dynamic LDS array of one bf16 per column and tensor; either way
+// every column belongs to exactly one thread, so no synchronisation is involved.
+template <int NCHW, int TENSORS>
+constexpr bool colmax_in_lds() { return NCHW * 4 * TENSORS > 32; }
+
 }  // namespace l8

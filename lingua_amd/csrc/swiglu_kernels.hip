@@ -28,12 +28,6 @@ namespace l8 {
 constexpr int kGateBlock = 256;
 constexpr int kGateWaves = kGateBlock / 64;
 
-L8_DEV uint32_t bf16_rne_bits(float v) {
-  const __bf16 b = (__bf16)v;
-  return (uint32_t) __builtin_bit_cast(unsigned short, b);
-}
-L8_DEV float bf16_round(float v) { return bf16_bits_to_f32(bf16_rne_bits(v)); }
-
 // 1 / (1 + exp(-x)) with the hardware exp2 and reciprocal (about 1 ulp of fp32
 // each).  The library exp and the IEEE division cost ~5x the instructions and
 // made these kernels VALU-bound (302 us forward / 550 us backward on
@@ -71,27 +65,6 @@ L8_DEV void gate_bwd2(uint32_t d, uint32_t a, uint32_t b, uint32_t &g1, uint32_t
   g1 = g1l | (g1h << 16);
   g3 = g3l | (g3h << 16);
 }
-
-// amax bits (uniform) -> scale, 1/scale, finite flag, as in the row-wise cast
-struct RowScale {
-  float s, recip;
-  bool finite;
-};
-L8_DEV RowScale row_scale(uint32_t amax_bits) {
-  RowScale r;
-  r.finite = amax_bits < 0x7f80u;
-  r.s = r.finite ? scale_from_amax(bf16_bits_to_f32(amax_bits))
-                 : __uint_as_float(amax_bits == 0x7f80u ? 0x7f800000u : 0x7fc00000u);
-  r.recip = recip_exact(r.s);
-  return r;
-}
-
-// Column maxima live in registers (packed pairs, NCHW * 4 dwords per tensor)
-// while that fits the 256-register budget of two workgroups per CU, else in a
-// dynamic LDS array of one bf16 per column and tensor; either way every column
-// belongs to exactly one thread, so no synchronisation is involved.
-template <int NCHW, int TENSORS>
-constexpr bool colmax_in_lds() { return NCHW * 4 * TENSORS > 32; }
 
 template <int NCHW, bool COLMAX>
 __global__ __launch_bounds__(kGateBlock, 2) void swiglu_cast_rowwise_kernel(

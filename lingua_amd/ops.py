@@ -247,3 +247,34 @@ def swiglu_bwd_cast_rowwise(dh: torch.Tensor, h1: torch.Tensor, h3: torch.Tensor
             ws.data_ptr() if ws is not None else None, ws_bytes, st)
     _lib.check(code, "l8_swiglu_bwd_cast_rowwise")
     return g1, g3, q1, q3, s1, s3
+
+
+def rmsnorm_cast_rowwise(x: torch.Tensor, weight: torch.Tensor, eps: float, want_q: bool = True,
+                         col_amax: Optional[torch.Tensor] = None, want_rstd: bool = True):
+    """y = bf16((f32(x) * rsqrt(mean(x^2) + eps)) * f32(weight)) and its row-wise cast in one pass.
+    Returns (y [R,C] bf16, q [R,C] fp8 | None, scale [R,1] fp32 | None, rstd [R,1] fp32 | None)."""
+    x = _rows_2d(x, torch.bfloat16, "rmsnorm_cast_rowwise")
+    st = _prep(x, "rmsnorm_cast_rowwise")
+    R, C = x.shape
+    dev = x.device
+    if weight.dtype not in (torch.bfloat16, torch.float32) or weight.numel() != C or weight.device != dev:
+        raise RuntimeError("rmsnorm_cast_rowwise: weight must be bf16 or fp32 with C elements on the same device")
+    weight = weight.contiguous()
+    if col_amax is not None and (not want_q or col_amax.dtype != torch.float32 or col_amax.numel() != C or not col_amax.is_contiguous()):
+        raise RuntimeError("rmsnorm_cast_rowwise: col_amax needs the cast and must be a contiguous fp32 tensor with C elements")
+    y = torch.empty((R, C), dtype=torch.bfloat16, device=dev)
+    q = torch.empty((R, C), dtype=torch.float8_e4m3fn, device=dev) if want_q else None
+    scale = torch.empty((R, 1), dtype=torch.float32, device=dev) if want_q else None
+    rstd = torch.empty((R, 1), dtype=torch.float32, device=dev) if want_rstd else None
+    ws, ws_bytes = None, 0
+    if col_amax is not None:
+        ws_bytes = _lib.load().l8_rmsnorm_workspace(R, C)
+        ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev) if ws_bytes else None
+    with _timed("rmsnorm_cast_rowwise", R * C * (4 + (1 if want_q else 0)) + 8 * R, dev):
+        code = _lib.load().l8_rmsnorm_cast_rowwise(
+            x.data_ptr(), weight.data_ptr(), int(weight.dtype == torch.float32), R, C, _ld(x), float(eps), y.data_ptr(), C,
+            q.data_ptr() if want_q else None, C, scale.data_ptr() if want_q else None,
+            rstd.data_ptr() if want_rstd else None, col_amax.data_ptr() if col_amax is not None else None,
+            ws.data_ptr() if ws is not None else None, ws_bytes, st)
+    _lib.check(code, "l8_rmsnorm_cast_rowwise")
+    return y, q, scale, rstd

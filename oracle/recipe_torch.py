@@ -84,6 +84,13 @@ def linear_fwd_bwd(a, b_t, grad_out, bias=None, wgrad_fp8=True):
     return out, grad_a, grad_b, grad_bias
 
 
+def rmsnorm(x: torch.Tensor, weight: torch.Tensor, eps: float) -> torch.Tensor:
+    """lingua/transformer.py:283-289: ``_norm(x.float()) * weight.float()`` cast back to x's dtype."""
+    xf = x.float()
+    out = xf * torch.rsqrt((xf * xf).mean(-1, keepdim=True) + eps)
+    return (out * weight.float()).type_as(x)
+
+
 def swiglu_gate(h1: torch.Tensor, h3: torch.Tensor) -> torch.Tensor:
     """lingua/transformer.py:469-471 between the linears: ``F.silu(h1) * h3`` as eager
     PyTorch runs it on bf16 tensors (silu in fp32 rounded to bf16, then a bf16 multiply)."""

@@ -196,3 +196,20 @@ def test_swiglu_gate_oracle_against_float64_closed_forms():
     g1z, g3z = rt.swiglu_gate_bwd(one, z, one)
     assert g1z[0, :2].tolist() == [0.5, 1.0] and abs(float(g1z[0, 2])) < 1e-14
     assert g3z[0, :2].tolist() == [0.0, 40.0]
+
+
+def test_rmsnorm_oracle_against_float64():
+    """oracle.recipe_torch.rmsnorm is the reference's eager op chain; pin it against x / sqrt(mean(x^2) + eps) * w
+    in float64 (one bf16 rounding at the end: half an ulp = 2^-8 relative, plus fp32 noise)."""
+    g = torch.Generator().manual_seed(78)
+    x = (torch.randn((48, 320), generator=g) * 4).to(torch.bfloat16)
+    w = (1 + 0.2 * torch.randn(320, generator=g)).to(torch.bfloat16)
+    y = rt.rmsnorm(x, w, 1e-5)
+    xd = x.double()
+    want = xd / torch.sqrt((xd * xd).mean(-1, keepdim=True) + 1e-5) * w.double()
+    assert y.dtype == torch.bfloat16
+    assert float(((y.double() - want).abs() / want.abs().clamp_min(1e-30)).max()) <= 2.0 ** -7.99
+    # a constant row c normalises to sign(c) * w (for |c| >> sqrt(eps)); a zero row stays zero
+    z = torch.full((1, 64), -3.0, dtype=torch.bfloat16)
+    assert torch.equal(rt.rmsnorm(z, torch.ones(64, dtype=torch.bfloat16), 1e-6), torch.full((1, 64), -1.0, dtype=torch.bfloat16))
+    assert float(rt.rmsnorm(torch.zeros((1, 64), dtype=torch.bfloat16), torch.ones(64), 1e-6).abs().max()) == 0.0
