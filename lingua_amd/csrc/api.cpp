@@ -18,8 +18,12 @@ int fail(int code, const char *fmt, ...) {
   return code;
 }
 
-constexpr int kMaxDev = 64;
 static int g_cus[kMaxDev];  // 0 = not queried yet; benign race: every thread writes the same value
+
+int device_slot() {
+  int dev = 0;
+  return (hipGetDevice(&dev) == hipSuccess && dev >= 0 && dev < kMaxDev) ? dev : -1;
+}
 
 int num_cus() {
   int dev = 0;

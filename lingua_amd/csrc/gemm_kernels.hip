@@ -566,10 +566,11 @@ extern "C" int l8_gemm_nt(const void *A, const void *B, int64_t M, int64_t N, in
   p.tiles_n = (int)((N + al.bn - 1) / al.bn);
   const int64_t nblocks = (int64_t)p.tiles_m * p.tiles_n;
   L8_REQUIRE(nblocks < (1LL << 31), "l8_gemm_nt: too many tiles");
-  static bool attr_done[kNumAlgos] = {};
-  if (!attr_done[algo - 1]) {  // idempotent; a race only repeats the call
+  static bool attr_done[kMaxDev][kNumAlgos] = {};  // idempotent; a race only repeats the call
+  const int slot = device_slot();
+  if (slot < 0 || !attr_done[slot][algo - 1]) {
     L8_HIP(hipFuncSetAttribute((const void *)al.fn, hipFuncAttributeMaxDynamicSharedMemorySize, al.lds));
-    attr_done[algo - 1] = true;
+    if (slot >= 0) attr_done[slot][algo - 1] = true;
   }
   hipLaunchKernelGGL(al.fn, dim3((unsigned)nblocks), dim3(al.threads), al.lds, (hipStream_t)stream, p);
   L8_HIP(hipGetLastError());

@@ -27,6 +27,11 @@ int fail(int code, const char *fmt, ...);  // records the thread-local message, 
 
 int num_cus();  // compute units of the current device (cached per device)
 
+// Per-device one-time set-up (function attributes are per device): index of the
+// current device into tables of kMaxDev entries, or -1 (then nothing is cached).
+constexpr int kMaxDev = 64;
+int device_slot();
+
 // Folds partial column maxima [slots, C] (bf16, one row per workgroup of a
 // row-wise kernel) into col_amax[C] (fp32 bit patterns, max-merged).  Defined in cast_kernels.hip.
 int fold_colmax(const void *partials, int64_t slots, int64_t C, float *col_amax, hipStream_t st);

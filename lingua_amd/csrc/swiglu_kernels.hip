@@ -282,9 +282,11 @@ static int launch_fwd(const void *h1, const void *h3, int64_t R, int64_t C, int6
   if (col_amax) {
     const size_t lds = colmax_in_lds<NCHW, 1>() ? (size_t)C * 2 : 0;
     if (lds > 48 * 1024) {  // above the default limit for dynamic LDS; idempotent
-      static bool raised = false;
-      if (!raised) L8_HIP(hipFuncSetAttribute((const void *)swiglu_cast_rowwise_kernel<NCHW, true>, hipFuncAttributeMaxDynamicSharedMemorySize, 64 * 1024));
-      raised = true;
+      static bool raised[kMaxDev] = {};
+      const int slot = device_slot();
+      if (slot < 0 || !raised[slot])
+        L8_HIP(hipFuncSetAttribute((const void *)swiglu_cast_rowwise_kernel<NCHW, true>, hipFuncAttributeMaxDynamicSharedMemorySize, 64 * 1024));
+      if (slot >= 0) raised[slot] = true;
     }
     hipLaunchKernelGGL((swiglu_cast_rowwise_kernel<NCHW, true>), dim3((unsigned)blocks), dim3(kGateBlock), lds, st,
                        (const uint16_t *)h1, (const uint16_t *)h3, R, (int)C, ld1, ld3, (uint16_t *)h, ldh, (uint8_t *)q, ldq,
@@ -308,9 +310,11 @@ static int launch_bwd(const void *dh, const void *h1, const void *h3, int64_t R,
     uint16_t *w1 = (uint16_t *)ws, *w3 = w1 + blocks * C;
     const size_t lds = colmax_in_lds<NCHW, 2>() ? (size_t)C * 4 : 0;
     if (lds > 48 * 1024) {  // above the default limit for dynamic LDS; idempotent
-      static bool raised = false;
-      if (!raised) L8_HIP(hipFuncSetAttribute((const void *)swiglu_bwd_cast_rowwise_kernel<NCHW, true>, hipFuncAttributeMaxDynamicSharedMemorySize, 64 * 1024));
-      raised = true;
+      static bool raised[kMaxDev] = {};
+      const int slot = device_slot();
+      if (slot < 0 || !raised[slot])
+        L8_HIP(hipFuncSetAttribute((const void *)swiglu_bwd_cast_rowwise_kernel<NCHW, true>, hipFuncAttributeMaxDynamicSharedMemorySize, 64 * 1024));
+      if (slot >= 0) raised[slot] = true;
     }
     hipLaunchKernelGGL((swiglu_bwd_cast_rowwise_kernel<NCHW, true>), dim3((unsigned)blocks), dim3(kGateBlock), lds, st,
                        (const uint16_t *)dh, (const uint16_t *)h1, (const uint16_t *)h3, R, (int)C, lddh, ld1, ld3,
