@@ -53,6 +53,10 @@ class Fp8Config:
     # (w1 / w3 of the MLP, wq / wk / wv of attention) quantise it once per
     # forward and once per backward instead of once each
     share_input_casts: bool = True
+    # route Fp8Linear through the torch.library operators of lingua_amd.custom_ops
+    # (opaque to torch.compile, nameable in activation-checkpointing policies)
+    # instead of the plain autograd.Function
+    use_custom_ops: bool = False
 
 
 config = Fp8Config()
@@ -120,29 +124,80 @@ _fwd_cast = _LastCast()   # a -> (qa, sa, a_col_amax | None)
 _bwd_cast = _LastCast()   # a -> (qat, sat)
 
 
+def linear_forward(a, b_t, bias, need_wgrad_stats: bool, gemm_algo: int):
+    """Forward of lingua/float8.py:85-96 on 2-D bf16 operands.  Returns ``(out, amax_b_t, a_col_amax | None)``:
+    the two extra tensors are what backward needs beyond ``a`` and ``b_t``."""
+    if a.dtype != torch.bfloat16 or b_t.dtype != torch.bfloat16:
+        raise RuntimeError(f"Fp8LinearFn: bf16 input and weight required, got {a.dtype} and {b_t.dtype}")
+    # column amaxes of `a` fall out of the row-wise pass; wgrad wants them
+    _bwd_cast.clear()
+    hit = _fwd_cast.get(a, b_t.data_ptr()) if config.share_input_casts else None
+    if hit is not None and (hit[2] is not None or not need_wgrad_stats):
+        qa, sa, a_col_amax = hit
+        if not need_wgrad_stats:
+            a_col_amax = None
+    else:
+        a_col_amax = torch.zeros(a.shape[1], dtype=torch.float32, device=a.device) if need_wgrad_stats else None
+        qa, sa, _ = ops.cast_rowwise(a, col_amax=a_col_amax)
+        if config.share_input_casts:
+            _fwd_cast.put(a, (qa, sa, a_col_amax), b_t.data_ptr())
+    qb, sb, amax_b_t = ops.cast_rowwise(b_t)
+    out = ops.gemm_nt(qa, qb, sa, sb, bias, algo=gemm_algo)
+    return out, amax_b_t, a_col_amax
+
+
+def linear_backward(grad_out, a, b_t, amax_b_t, a_col_amax, need_a: bool, need_b: bool, need_bias: bool,
+                    fp8_wgrad: bool, gemm_algo: int):
+    """Backward of lingua/float8.py:99-131 (fp8 wgrad optional).  Returns ``(grad_a, grad_b, grad_bias)`` with
+    ``None`` where not needed."""
+    if grad_out.dtype != torch.bfloat16:
+        raise RuntimeError(f"Fp8LinearFn.backward: bf16 grad_out required, got {grad_out.dtype}")
+    fp8_wgrad = fp8_wgrad and need_b
+    _fwd_cast.clear()
+
+    g_col_amax = None
+    if need_a:
+        # grad_out row-wise, weight tensor-wise from the row amaxes saved in
+        # forward, quantised straight into the [K,N] layout dgrad multiplies with
+        g_col_amax = torch.zeros(grad_out.shape[1], dtype=torch.float32, device=grad_out.device) if fp8_wgrad else None
+        qg, sg, _ = ops.cast_rowwise(grad_out, col_amax=g_col_amax)
+        amax_b = ops.amax_reduce(amax_b_t)
+        qb, sb = ops.cast_tensorwise(b_t, amax_b, transpose=True)
+        grad_a = ops.gemm_nt(qg, qb, sg, sb, None, algo=gemm_algo)
+    else:
+        grad_a = None
+
+    if need_b:
+        if fp8_wgrad:
+            if g_col_amax is None:
+                g_col_amax = ops.col_amax(grad_out)
+            qgt, sgt = ops.cast_colwise_transposed(grad_out, g_col_amax)
+            hit = _bwd_cast.get(a, b_t.data_ptr()) if config.share_input_casts else None
+            if hit is not None:
+                qat, sat = hit
+            else:
+                if a_col_amax is None:
+                    a_col_amax = ops.col_amax(a)
+                qat, sat = ops.cast_colwise_transposed(a, a_col_amax)
+                if config.share_input_casts:
+                    _bwd_cast.put(a, (qat, sat), b_t.data_ptr())
+            grad_b = ops.gemm_nt(qgt, qat, sgt, sat, None, algo=gemm_algo)
+        else:
+            grad_b = grad_out.t() @ a
+    else:
+        grad_b = None
+
+    grad_bias = grad_out.sum(dim=0) if need_bias else None
+    return grad_a, grad_b, grad_bias
+
+
 class Fp8LinearFn(torch.autograd.Function):
     """``out = a @ b_t.T + bias`` with fp8 operands (lingua/float8.py:83-131)."""
 
     @staticmethod
     def forward(ctx, a, b_t, bias):
-        if a.dtype != torch.bfloat16 or b_t.dtype != torch.bfloat16:
-            raise RuntimeError(f"Fp8LinearFn: bf16 input and weight required, got {a.dtype} and {b_t.dtype}")
         need_wgrad_stats = config.fp8_wgrad and b_t.requires_grad
-        # column amaxes of `a` fall out of the row-wise pass; wgrad wants them
-        _bwd_cast.clear()
-        hit = _fwd_cast.get(a, b_t.data_ptr()) if config.share_input_casts else None
-        if hit is not None and (hit[2] is not None or not need_wgrad_stats):
-            qa, sa, a_col_amax = hit
-            if not need_wgrad_stats:
-                a_col_amax = None
-        else:
-            a_col_amax = torch.zeros(a.shape[1], dtype=torch.float32, device=a.device) if need_wgrad_stats else None
-            qa, sa, _ = ops.cast_rowwise(a, col_amax=a_col_amax)
-            if config.share_input_casts:
-                _fwd_cast.put(a, (qa, sa, a_col_amax), b_t.data_ptr())
-        qb, sb, amax_b_t = ops.cast_rowwise(b_t)
-        out = ops.gemm_nt(qa, qb, sa, sb, bias, algo=config.gemm_algo)
-
+        out, amax_b_t, a_col_amax = linear_forward(a, b_t, bias, need_wgrad_stats, config.gemm_algo)
         ctx.a_requires_grad = a.requires_grad
         ctx.b_requires_grad = b_t.requires_grad
         ctx.bias_requires_grad = bias.requires_grad if bias is not None else False
@@ -162,55 +217,17 @@ class Fp8LinearFn(torch.autograd.Function):
         else:
             a, b_t, amax_b_t = ctx.saved_tensors
             a_col_amax = None
-        if grad_out.dtype != torch.bfloat16:
-            raise RuntimeError(f"Fp8LinearFn.backward: bf16 grad_out required, got {grad_out.dtype}")
-        fp8_wgrad = ctx.fp8_wgrad and ctx.b_requires_grad
-        _fwd_cast.clear()
-
-        qg = sg = None
-        g_col_amax = None
-        if ctx.a_requires_grad:
-            # grad_out row-wise, weight tensor-wise from the row amaxes saved in
-            # forward, quantised straight into the [K,N] layout dgrad multiplies with
-            g_col_amax = torch.zeros(grad_out.shape[1], dtype=torch.float32, device=grad_out.device) if fp8_wgrad else None
-            qg, sg, _ = ops.cast_rowwise(grad_out, col_amax=g_col_amax)
-            amax_b = ops.amax_reduce(amax_b_t)
-            qb, sb = ops.cast_tensorwise(b_t, amax_b, transpose=True)
-            grad_a = ops.gemm_nt(qg, qb, sg, sb, None, algo=ctx.gemm_algo)
-        else:
-            grad_a = None
-
-        if ctx.b_requires_grad:
-            if fp8_wgrad:
-                if g_col_amax is None:
-                    g_col_amax = ops.col_amax(grad_out)
-                qgt, sgt = ops.cast_colwise_transposed(grad_out, g_col_amax)
-                hit = _bwd_cast.get(a, b_t.data_ptr()) if config.share_input_casts else None
-                if hit is not None:
-                    qat, sat = hit
-                else:
-                    if a_col_amax is None:
-                        a_col_amax = ops.col_amax(a)
-                    qat, sat = ops.cast_colwise_transposed(a, a_col_amax)
-                    if config.share_input_casts:
-                        _bwd_cast.put(a, (qat, sat), b_t.data_ptr())
-                grad_b = ops.gemm_nt(qgt, qat, sgt, sat, None, algo=ctx.gemm_algo)
-            else:
-                grad_b = grad_out.t() @ a
-        else:
-            grad_b = None
-
-        if ctx.bias_requires_grad:
-            grad_bias = grad_out.sum(dim=0)
-        else:
-            grad_bias = None
-
-        return grad_a, grad_b, grad_bias
+        return linear_backward(grad_out, a, b_t, amax_b_t, a_col_amax, ctx.a_requires_grad, ctx.b_requires_grad,
+                               ctx.bias_requires_grad, ctx.fp8_wgrad, ctx.gemm_algo)
 
 
 class Fp8Linear(torch.nn.Linear):
     def forward(self, input: torch.Tensor) -> torch.Tensor:
-        out = Fp8LinearFn.apply(input.flatten(end_dim=-2), self.weight, self.bias)
+        if config.use_custom_ops:
+            from .custom_ops import fp8_linear
+            out = fp8_linear(input.flatten(end_dim=-2), self.weight, self.bias)
+        else:
+            out = Fp8LinearFn.apply(input.flatten(end_dim=-2), self.weight, self.bias)
         out = out.unflatten(0, input.shape[:-1])
         return out
 

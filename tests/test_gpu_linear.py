@@ -295,3 +295,42 @@ def test_linears_on_the_same_activation_share_its_casts():
         yb = l3(x)
         yc = l3(x / 1.0)
     assert torch.equal(yb, yc) and not torch.equal(ya, yb)
+
+
+def test_custom_ops_route_equals_the_autograd_function_and_compiles():
+    """config.use_custom_ops: same bits as the plain autograd.Function; the converted model traces as one graph
+    (aot_eager: fake tensors + functionalisation + the registered autograd formula, no code generation)."""
+    from lingua_amd import convert_linears_to_fp8, float8
+    from lingua_amd import custom_ops
+    from lingua_amd.callers import FeedForward
+    torch.manual_seed(6)
+    holder = nn.ModuleDict({"feed_forward": FeedForward(256, 512).to(device="cuda", dtype=torch.bfloat16)})
+    model = convert_linears_to_fp8(holder, "rowwise", r"feed_forward\.")["feed_forward"]
+    x = seeded_bf16((3, 32, 256), seed=31).cuda()
+    gy = seeded_bf16((3, 32, 256), std=0.02, seed=32).cuda()
+
+    def run(fn):
+        for p in model.parameters():
+            p.grad = None
+        xi = x.clone().requires_grad_(True)
+        y = fn(xi)
+        y.backward(gy)
+        return [y.detach(), xi.grad] + [p.grad.clone() for p in model.parameters()]
+
+    want = run(model)
+    old = float8.config.use_custom_ops
+    float8.config.use_custom_ops = True
+    try:
+        got = run(model)
+        compiled = torch.compile(model, backend="aot_eager", fullgraph=True)
+        got_compiled = run(compiled)
+        # the operators are addressable by name (what a checkpointing policy lists)
+        assert torch.ops.lingua_amd.fp8_linear_fwd.default is not None
+        torch.library.opcheck(custom_ops.fp8_linear_fwd, (x.flatten(0, 1), model.w1.weight.detach(), None, True, 0),
+                              test_utils=("test_schema", "test_faketensor"))
+    finally:
+        float8.config.use_custom_ops = old
+    for a, b in zip(got, want):
+        assert torch.equal(a.view(torch.int16), b.view(torch.int16))
+    for a, b in zip(got_compiled, want):
+        assert rel_l2(a, b) <= 1e-6

@@ -144,3 +144,21 @@ def test_public_names_match_reference_module():
     for name in ("EPS", "scale", "matmul", "Fp8LinearFn", "Fp8Linear", "named_replace", "convert_linears_to_fp8"):
         assert hasattr(lingua_amd, name)
     assert lingua_amd.EPS == 1e-12
+
+
+def test_custom_op_fake_kernels_on_meta_tensors():
+    """lingua_amd.custom_ops: shape-only implementations (what torch.compile traces with) need no GPU."""
+    import torch
+    from lingua_amd import custom_ops  # noqa: F401  (registers the operators)
+    a = torch.empty((32, 64), dtype=torch.bfloat16, device="meta")
+    w = torch.empty((48, 64), dtype=torch.bfloat16, device="meta")
+    bias = torch.empty((48,), dtype=torch.bfloat16, device="meta")
+    out, amax_w, col = torch.ops.lingua_amd.fp8_linear_fwd(a, w, bias, True, 0)
+    assert out.shape == (32, 48) and out.dtype == torch.bfloat16
+    assert amax_w.shape == (48, 1) and amax_w.dtype == torch.bfloat16
+    assert col.shape == (64,) and col.dtype == torch.float32
+    assert torch.ops.lingua_amd.fp8_linear_fwd(a, w, None, False, 0)[2].numel() == 0
+    ga, gb, gbias = torch.ops.lingua_amd.fp8_linear_bwd(out, a, w, amax_w, col, True, True, True, True, 0)
+    assert ga.shape == a.shape and gb.shape == w.shape and gbias.shape == (48,)
+    ga, gb, gbias = torch.ops.lingua_amd.fp8_linear_bwd(out, a, w, amax_w, col, False, True, False, True, 0)
+    assert ga.numel() == 0 and gb.shape == w.shape and gbias.numel() == 0
