@@ -40,8 +40,9 @@ def parse():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-sample-tokens", type=int, default=16384)
     ap.add_argument("--no-kernel-timing", action="store_true", help="do not record per-kernel events in the timed steps")
-    ap.add_argument("--workload", choices=["mlp7b", "llama1b"], default="mlp7b",
-                    help="mlp7b = the headline workload; llama1b = full Llama-1B-shaped forward+backward step "
+    ap.add_argument("--workload", choices=["mlp7b", "linear7b", "llama1b"], default="mlp7b",
+                    help="mlp7b = the headline workload; linear7b = one 4096->11008 Fp8Linear forward+backward on 16384 "
+                         "tokens (casts included); llama1b = full Llama-1B-shaped forward+backward step "
                          "(25 layers, dim 2048, ffn 8192, vocab 128256, 4 x 4096 tokens), reported in tokens/s")
     ap.add_argument("--no-extras", action="store_true",
                     help="skip the two side measurements: the fused-SwiGLU variant of the same MLP and "
@@ -138,6 +139,38 @@ def extras(torch, mlp, timed, args):
         res["torch_scaled_mm"] = None
         res["torch_scaled_mm_error"] = str(exc)[:200]
     return res
+
+
+def run_linear7b(args, torch, dev):
+    """One Fp8Linear 4096 -> 11008 on 16384 tokens, forward + backward (dgrad + fp8 wgrad), casts included."""
+    from lingua_amd import Fp8Linear
+    g = torch.Generator().manual_seed(0)
+    lin = Fp8Linear(DIM, FFN, bias=False, device=dev, dtype=torch.bfloat16)
+    with torch.no_grad():
+        lin.weight.copy_((torch.randn(FFN, DIM, generator=g) * 0.02).to(torch.bfloat16))
+    x = torch.randn(TOKENS, DIM, generator=g).to(torch.bfloat16).to(dev).requires_grad_(True)
+    gy = (torch.randn(TOKENS, FFN, generator=g) * 1e-2).to(torch.bfloat16).to(dev)
+
+    def step():
+        lin.weight.grad = x.grad = None
+        lin(x).backward(gy)
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    dt = (time.perf_counter() - t0) / args.steps
+    flop = 6 * TOKENS * DIM * FFN
+    print(json.dumps({
+        "metric": "fp8 rowwise linear fwd+bwd TFLOP/s, one 4096->11008 linear", "value": round(flop / dt / 1e12, 2),
+        "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(dt * 1e3, 4),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "fp8_e4m3fn", "data": "synthetic",
+        "config": {"workload": "single Fp8Linear 4096->11008 fwd+bwd, 16384 tokens, casts included", "flop_per_step": flop},
+        "frac_of_fp8_peak": round(flop / dt / 1e12 / PEAK_FP8_TFLOPS, 4),
+    }))
 
 
 def run_llama1b(args, torch, dev):
@@ -265,6 +298,9 @@ def main():
 
     if args.workload == "llama1b":
         run_llama1b(args, torch, dev)
+        return
+    if args.workload == "linear7b":
+        run_linear7b(args, torch, dev)
         return
 
     mlp = make_mlp(torch, nn, DIM, FFN, dev)
