@@ -151,6 +151,17 @@ int l8_rmsnorm_cast_rowwise(const void *x, const void *w, int w_is_f32, int64_t 
                             float *col_amax, void *workspace, int64_t workspace_bytes, void *stream);
 int64_t l8_rmsnorm_workspace(int64_t R, int64_t C);
 
+/* Backward of that norm (what autograd derives from lingua/transformer.py:283-289), one pass over gy and x:
+ *   xhat = f32(x) * rstd;  gh = f32(gy) * f32(w)
+ *   gx = bf16( (gh - xhat * mean(gh * xhat)) * rstd )      [R,C] (ldgx)
+ *   gw = sum over rows of f32(gy) * xhat                    fp32 [C], summed in a fixed order
+ *   rstd fp32 [R] as written by l8_rmsnorm_cast_rowwise; workspace of l8_rmsnorm_bwd_workspace(R, C) bytes
+ * Requires C % 8 == 0, C <= 8192, every leading dimension % 8 == 0. */
+int l8_rmsnorm_bwd(const void *gy, const void *x, const void *w, int w_is_f32, const float *rstd,
+                   int64_t R, int64_t C, int64_t ldg, int64_t ldx, void *gx, int64_t ldgx, float *gw,
+                   void *workspace, int64_t workspace_bytes, void *stream);
+int64_t l8_rmsnorm_bwd_workspace(int64_t R, int64_t C);
+
 int l8_gemm_algo_count(void);
 /* human-readable description of tile configuration `algo` (1-based), or NULL */
 const char *l8_gemm_algo_name(int algo);

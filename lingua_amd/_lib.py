@@ -33,11 +33,13 @@ SIGNATURES = {
                                    _p, _i64, _p],
     "l8_rmsnorm_cast_rowwise": [_p, _p, _int, _i64, _i64, _i64, ctypes.c_float, _p, _i64, _p, _i64, _p, _p, _p, _p, _i64, _p],
     "l8_rmsnorm_workspace": [_i64, _i64],
+    "l8_rmsnorm_bwd": [_p, _p, _p, _int, _p, _i64, _i64, _i64, _i64, _p, _i64, _p, _p, _i64, _p],
+    "l8_rmsnorm_bwd_workspace": [_i64, _i64],
     "l8_gemm_algo_count": [],
     "l8_gemm_algo_name": [_int],
 }
 _RETURNS_STR = {"l8_last_error", "l8_gemm_algo_name"}
-_RETURNS_I64 = {"l8_cast_rowwise_workspace", "l8_swiglu_workspace", "l8_rmsnorm_workspace"}
+_RETURNS_I64 = {"l8_cast_rowwise_workspace", "l8_swiglu_workspace", "l8_rmsnorm_workspace", "l8_rmsnorm_bwd_workspace"}
 
 _lib = None
 _lock = threading.Lock()

@@ -153,6 +153,114 @@ __global__ __launch_bounds__(kNormBlock, 2) void rmsnorm_cast_rowwise_kernel(
   }
 }
 
+// Backward of the norm: with xhat = x * r and gh = gy * w,
+//   gx = (gh - xhat * mean(gh * xhat)) * r        (bf16)
+//   gw = sum over rows of gy * xhat               (fp32)
+// One workgroup per row again; the row products for gw are accumulated in
+// registers over all rows a workgroup sees and leave as one row of fp32
+// partial sums per workgroup, which rmsnorm_gw_fold_kernel adds up column by
+// column in a fixed order (no atomics: the result does not depend on timing).
+template <int NCHW, bool W_F32>
+__global__ __launch_bounds__(kNormBlock, 2) void rmsnorm_bwd_kernel(
+    const uint16_t *__restrict__ gy, const uint16_t *__restrict__ x, const void *__restrict__ w,
+    const float *__restrict__ rstd, int64_t R, int C, int64_t ldg, int64_t ldx, uint16_t *__restrict__ gx, int64_t ldgx,
+    float *__restrict__ gw_partials) {
+  __shared__ float red[2][kNormWaves];
+  const int lane = threadIdx.x & 63;
+  const int wave = threadIdx.x >> 6;
+  auto col_of = [&](int j) { return (j * kNormWaves + wave) * 512 + lane * 8; };
+  float wf[NCHW][8], gwacc[NCHW][8];
+#pragma unroll
+  for (int j = 0; j < NCHW; ++j) {
+    const int c = col_of(j);
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      gwacc[j][e] = 0.0f;
+      if (c < C) wf[j][e] = W_F32 ? ((const float *)w)[c + e] : bf16_bits_to_f32(((const uint16_t *)w)[c + e]);
+      else wf[j][e] = 0.0f;
+    }
+  }
+  const float inv_c = 1.0f / (float)C;
+  int it = 0;
+  for (int64_t r = blockIdx.x; r < R; r += gridDim.x, ++it) {
+    const float rinv = rstd[r];
+    float xh[NCHW][8], gh[NCHW][8];
+    float dot = 0.0f;
+#pragma unroll
+    for (int j = 0; j < NCHW; ++j) {
+      const int c = col_of(j);
+      v4i xv = {0, 0, 0, 0}, gv = {0, 0, 0, 0};
+      if (c < C) {
+        xv = __builtin_nontemporal_load((const v4i *)(x + r * ldx + c));
+        gv = __builtin_nontemporal_load((const v4i *)(gy + r * ldg + c));
+      }
+#pragma unroll
+      for (int k = 0; k < 4; ++k) {
+#pragma unroll
+        for (int half = 0; half < 2; ++half) {
+          const int e = 2 * k + half;
+          const float xe = __uint_as_float(half ? ((uint32_t)xv[k] & 0xffff0000u) : ((uint32_t)xv[k] << 16));
+          const float ge = __uint_as_float(half ? ((uint32_t)gv[k] & 0xffff0000u) : ((uint32_t)gv[k] << 16));
+          xh[j][e] = xe * rinv;
+          gh[j][e] = ge * wf[j][e];
+          gwacc[j][e] += ge * xh[j][e];
+          dot += gh[j][e] * xh[j][e];
+        }
+      }
+    }
+    dot = wave_sum_f32(dot);
+    if (lane == 0) red[it & 1][wave] = dot;
+    __syncthreads();
+    float tot = 0.0f;
+#pragma unroll
+    for (int wv = 0; wv < kNormWaves; ++wv) tot += red[it & 1][wv];
+    const float c1 = tot * inv_c;
+#pragma unroll
+    for (int j = 0; j < NCHW; ++j) {
+      const int c = col_of(j);
+      if (c < C) {
+        v4i out;
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+          const uint32_t lo = bf16_rne_bits((gh[j][2 * k] - xh[j][2 * k] * c1) * rinv);
+          const uint32_t hi = bf16_rne_bits((gh[j][2 * k + 1] - xh[j][2 * k + 1] * c1) * rinv);
+          out[k] = (int)(lo | (hi << 16));
+        }
+        __builtin_nontemporal_store(out, (v4i *)(gx + r * ldgx + c));
+      }
+    }
+  }
+#pragma unroll
+  for (int j = 0; j < NCHW; ++j) {
+    const int c = col_of(j);
+    if (c < C) {
+      float *dst = gw_partials + (int64_t)blockIdx.x * C + c;
+      *(v4f *)dst = v4f{gwacc[j][0], gwacc[j][1], gwacc[j][2], gwacc[j][3]};
+      *(v4f *)(dst + 4) = v4f{gwacc[j][4], gwacc[j][5], gwacc[j][6], gwacc[j][7]};
+    }
+  }
+}
+
+// gw[c] = sum over the partial rows.  A workgroup owns 32 columns; thread (tx, ty)
+// adds slots ty, ty+8, ... of column tx, then the eight sums are added in order of ty.
+__global__ __launch_bounds__(256) void rmsnorm_gw_fold_kernel(const float *__restrict__ partials, int n_slots, int C,
+                                                              float *__restrict__ gw) {
+  __shared__ float part[8][32];
+  const int tx = threadIdx.x & 31, ty = threadIdx.x >> 5;
+  const int c = blockIdx.x * 32 + tx;
+  float s = 0.0f;
+  if (c < C)
+    for (int sl = ty; sl < n_slots; sl += 8) s += partials[(int64_t)sl * C + c];
+  part[ty][tx] = s;
+  __syncthreads();
+  if (ty == 0 && c < C) {
+    float t = part[0][tx];
+#pragma unroll
+    for (int k = 1; k < 8; ++k) t += part[k][tx];
+    gw[c] = t;
+  }
+}
+
 static int64_t norm_blocks(int64_t R) {
   const int64_t cap = (int64_t)num_cus() * 2;
   return R < cap ? R : cap;
@@ -179,9 +287,60 @@ static int launch_norm(const void *x, const void *w, int64_t R, int64_t C, int64
   return L8_OK;
 }
 
+template <int NCHW, bool W_F32>
+static int launch_norm_bwd(const void *gy, const void *x, const void *w, const float *rstd, int64_t R, int64_t C,
+                           int64_t ldg, int64_t ldx, void *gx, int64_t ldgx, float *gw, void *ws, hipStream_t st) {
+  const int64_t blocks = norm_blocks(R);
+  hipLaunchKernelGGL((rmsnorm_bwd_kernel<NCHW, W_F32>), dim3((unsigned)blocks), dim3(kNormBlock), 0, st,
+                     (const uint16_t *)gy, (const uint16_t *)x, w, rstd, R, (int)C, ldg, ldx, (uint16_t *)gx, ldgx,
+                     (float *)ws);
+  L8_HIP(hipGetLastError());
+  hipLaunchKernelGGL(rmsnorm_gw_fold_kernel, dim3((unsigned)((C + 31) / 32)), dim3(256), 0, st, (const float *)ws,
+                     (int)blocks, (int)C, gw);
+  L8_HIP(hipGetLastError());
+  return L8_OK;
+}
+
 }  // namespace l8
 
 using namespace l8;
+
+extern "C" int64_t l8_rmsnorm_bwd_workspace(int64_t R, int64_t C) {
+  if (R <= 0 || C <= 0) return 0;
+  return norm_blocks(R) * C * (int64_t)sizeof(float);
+}
+
+extern "C" int l8_rmsnorm_bwd(const void *gy, const void *x, const void *w, int w_is_f32, const float *rstd, int64_t R,
+                              int64_t C, int64_t ldg, int64_t ldx, void *gx, int64_t ldgx, float *gw, void *workspace,
+                              int64_t workspace_bytes, void *stream) {
+  L8_REQUIRE(R >= 0 && C >= 0, "l8_rmsnorm_bwd: negative shape R=%lld C=%lld", (long long)R, (long long)C);
+  if (C == 0) return L8_OK;
+  L8_REQUIRE(gw, "l8_rmsnorm_bwd: null pointer");
+  if (R == 0) {  // no rows: gw = 0, written by the fold kernel over zero partial rows
+    hipLaunchKernelGGL(rmsnorm_gw_fold_kernel, dim3((unsigned)((C + 31) / 32)), dim3(256), 0, (hipStream_t)stream,
+                       (const float *)nullptr, 0, (int)C, gw);
+    L8_HIP(hipGetLastError());
+    return L8_OK;
+  }
+  L8_REQUIRE(gy && x && w && rstd && gx, "l8_rmsnorm_bwd: null pointer");
+  L8_REQUIRE(C % 8 == 0 && ldg % 8 == 0 && ldx % 8 == 0 && ldgx % 8 == 0 && ldg >= C && ldx >= C && ldgx >= C,
+             "l8_rmsnorm_bwd: C=%lld and the leading dimensions must be multiples of 8 with ld >= C", (long long)C);
+  L8_REQUIRE(((uintptr_t)gy % 16) == 0 && ((uintptr_t)x % 16) == 0 && ((uintptr_t)gx % 16) == 0,
+             "l8_rmsnorm_bwd: gy, x and gx must be 16-byte aligned");
+  L8_REQUIRE(C <= kNormMaxC, "l8_rmsnorm_bwd: C=%lld exceeds %lld", (long long)C, (long long)kNormMaxC);
+  const int64_t need = l8_rmsnorm_bwd_workspace(R, C);
+  L8_REQUIRE(workspace && workspace_bytes >= need && ((uintptr_t)workspace % 16) == 0,
+             "l8_rmsnorm_bwd: needs a 16-byte aligned workspace of %lld bytes", (long long)need);
+  hipStream_t st = (hipStream_t)stream;
+  const int64_t nchw = ((C + 511) / 512 + kNormWaves - 1) / kNormWaves;
+#define L8_NORM_BWD(N)                                                                                               \
+  return w_is_f32 ? launch_norm_bwd<N, true>(gy, x, w, rstd, R, C, ldg, ldx, gx, ldgx, gw, workspace, st)             \
+                  : launch_norm_bwd<N, false>(gy, x, w, rstd, R, C, ldg, ldx, gx, ldgx, gw, workspace, st)
+  if (nchw <= 1) L8_NORM_BWD(1);
+  if (nchw <= 2) L8_NORM_BWD(2);
+  L8_NORM_BWD(4);
+#undef L8_NORM_BWD
+}
 
 extern "C" int64_t l8_rmsnorm_workspace(int64_t R, int64_t C) {
   if (R <= 0 || C <= 0) return 0;

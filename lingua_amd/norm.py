@@ -2,7 +2,7 @@
 
 ``Fp8RMSNorm`` is a drop-in for the reference's ``RMSNorm``
 (lingua/transformer.py:264-292: ``(x.float() * rsqrt(mean(x^2) + eps) * weight.float()).type_as(x)``).
-Its forward is one kernel (``l8_rmsnorm_cast_rowwise``) that writes the bf16
+Its backward is one kernel too (``l8_rmsnorm_bwd``).  Its forward (``l8_rmsnorm_cast_rowwise``) writes the bf16
 output and, from the same registers, the row-wise fp8 copy that the linears
 fed by the norm (wq / wk / wv, w1 / w3) would otherwise each compute in a pass
 of their own (lingua/float8.py:86-87, :43-47).  The quantised copy is handed
@@ -36,15 +36,11 @@ class Fp8RMSNormFn(torch.autograd.Function):
     @staticmethod
     def backward(ctx, gy):
         x2d, weight, rstd = ctx.saved_tensors
-        gyf = gy.flatten(end_dim=-2).float()
-        xhat = x2d.float() * rstd
-        gw = gx = None
-        if ctx.needs_input_grad[1]:
-            gw = (gyf * xhat).sum(dim=0).to(weight.dtype)
-        if ctx.needs_input_grad[0]:
-            gxhat = gyf * weight.float()
-            gx = ((gxhat - xhat * (gxhat * xhat).mean(dim=-1, keepdim=True)) * rstd).to(x2d.dtype).reshape(ctx.x_shape)
-        return gx, gw, None, None
+        if gy.dtype != torch.bfloat16:
+            raise RuntimeError(f"Fp8RMSNorm.backward: bf16 grad_out required, got {gy.dtype}")
+        gx2d, gw = ops.rmsnorm_bwd(gy.flatten(end_dim=-2), x2d, weight, rstd)
+        gx = gx2d.reshape(ctx.x_shape) if ctx.needs_input_grad[0] else None
+        return gx, (gw.to(weight.dtype) if ctx.needs_input_grad[1] else None), None, None
 
 
 class Fp8RMSNorm(torch.nn.Module):

@@ -278,3 +278,29 @@ def rmsnorm_cast_rowwise(x: torch.Tensor, weight: torch.Tensor, eps: float, want
             ws.data_ptr() if ws is not None else None, ws_bytes, st)
     _lib.check(code, "l8_rmsnorm_cast_rowwise")
     return y, q, scale, rstd
+
+
+def rmsnorm_bwd(gy: torch.Tensor, x: torch.Tensor, weight: torch.Tensor, rstd: torch.Tensor):
+    """Backward of the RMSNorm: returns (gx [R,C] bf16, gw [C] fp32) from gy, x (bf16 [R,C]), weight [C], rstd [R,1] fp32."""
+    gy = _rows_2d(gy, torch.bfloat16, "rmsnorm_bwd(gy)")
+    x = _rows_2d(x, torch.bfloat16, "rmsnorm_bwd(x)")
+    if gy.shape != x.shape or gy.device != x.device:
+        raise RuntimeError("rmsnorm_bwd: gy and x must have the same shape and device")
+    st = _prep(x, "rmsnorm_bwd")
+    R, C = x.shape
+    dev = x.device
+    if weight.dtype not in (torch.bfloat16, torch.float32) or weight.numel() != C or weight.device != dev:
+        raise RuntimeError("rmsnorm_bwd: weight must be bf16 or fp32 with C elements on the same device")
+    if rstd.dtype != torch.float32 or rstd.numel() != R or rstd.device != dev:
+        raise RuntimeError("rmsnorm_bwd: rstd must be fp32 with R elements on the same device")
+    weight, rstd = weight.contiguous(), rstd.contiguous()
+    gx = torch.empty((R, C), dtype=torch.bfloat16, device=dev)
+    gw = torch.empty((C,), dtype=torch.float32, device=dev)
+    ws_bytes = _lib.load().l8_rmsnorm_bwd_workspace(R, C)
+    ws = torch.empty(max(ws_bytes, 16), dtype=torch.uint8, device=dev)
+    with _timed("rmsnorm_bwd", R * C * 6 + 4 * R, dev):
+        code = _lib.load().l8_rmsnorm_bwd(gy.data_ptr(), x.data_ptr(), weight.data_ptr(), int(weight.dtype == torch.float32),
+                                          rstd.data_ptr(), R, C, _ld(gy), _ld(x), gx.data_ptr(), C, gw.data_ptr(),
+                                          ws.data_ptr(), ws_bytes, st)
+    _lib.check(code, "l8_rmsnorm_bwd")
+    return gx, gw
