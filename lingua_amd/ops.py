@@ -135,6 +135,10 @@ def cast_colwise_transposed(x: torch.Tensor, col_amax_f32: torch.Tensor, pad_to:
     R, C = x.shape
     if col_amax_f32.dtype != torch.float32 or col_amax_f32.numel() != C or not col_amax_f32.is_contiguous():
         raise RuntimeError("cast_colwise_transposed: col_amax must be a contiguous fp32 tensor with C elements")
+    if R == 0:
+        # no rows: the product over them is zero; one block of zero columns keeps the GEMM's reduction length valid
+        q = torch.zeros((C, pad_to), dtype=torch.uint8, device=x.device).view(torch.float8_e4m3fn)
+        return q, (torch.clamp(col_amax_f32, min=1e-12) / 448.0).reshape(C, 1)
     Rp = (R + pad_to - 1) // pad_to * pad_to
     if Rp == R:
         q = torch.empty((C, R), dtype=torch.float8_e4m3fn, device=x.device)

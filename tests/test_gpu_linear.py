@@ -334,3 +334,27 @@ def test_custom_ops_route_equals_the_autograd_function_and_compiles():
         assert torch.equal(a.view(torch.int16), b.view(torch.int16))
     for a, b in zip(got_compiled, want):
         assert rel_l2(a, b) <= 1e-6
+
+
+def test_empty_batch_and_single_token():
+    """Zero tokens (an empty micro-batch) and one token go through forward and backward: outputs of the right
+    shape, zero weight gradient for the empty batch, oracle parity for the single token."""
+    from lingua_amd import Fp8Linear
+    torch.manual_seed(8)
+    lin = Fp8Linear(128, 256, bias=True, device="cuda", dtype=torch.bfloat16)
+    x0 = torch.zeros((0, 128), dtype=torch.bfloat16, device="cuda", requires_grad=True)
+    y0 = lin(x0)
+    assert y0.shape == (0, 256)
+    y0.backward(torch.zeros_like(y0))
+    assert x0.grad.shape == (0, 128)
+    assert float(lin.weight.grad.float().abs().max()) == 0.0 and float(lin.bias.grad.float().abs().max()) == 0.0
+    lin.weight.grad = lin.bias.grad = None
+    x1 = seeded_bf16((1, 128), seed=41).cuda().requires_grad_(True)
+    g1 = seeded_bf16((1, 256), std=0.02, seed=42).cuda()
+    y1 = lin(x1)
+    y1.backward(g1)
+    W, b = lin.weight.detach().cpu(), lin.bias.detach().cpu()
+    assert rel_l2(y1, oracle.linear_forward(x1.detach().cpu(), W, b)) <= TOL
+    assert rel_l2(x1.grad, oracle.linear_dgrad(g1.cpu(), W)) <= TOL
+    assert rel_l2(lin.weight.grad, oracle.linear_wgrad_fp8(g1.cpu(), x1.detach().cpu())) <= TOL
+    assert torch.equal(lin.bias.grad, g1[0])
