@@ -205,6 +205,18 @@ def test_fused_mlp_partial_requires_grad():
     assert rel_l2(fused.w2.weight.grad, plain.w2.weight.grad) <= TOL
 
 
+def test_fused_mlp_with_no_tokens():
+    plain, fused = _mlps(256, 512, seed=10)
+    x = torch.zeros((0, 256), dtype=torch.bfloat16, device="cuda", requires_grad=True)
+    y = fused(x)
+    assert y.shape == (0, 256)
+    y.backward(torch.zeros_like(y))
+    assert x.grad.shape == (0, 256)
+    for n in ("w1", "w2", "w3"):
+        g = getattr(fused, n).weight.grad
+        assert g.shape == getattr(fused, n).weight.shape and float(g.float().abs().max()) == 0.0
+
+
 def test_fuse_feed_forward_rejects_other_modules():
     from lingua_amd.swiglu import fuse_feed_forward
     m = torch.nn.Module()
