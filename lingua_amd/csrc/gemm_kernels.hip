@@ -36,8 +36,9 @@
 //     the LDS side of a direct load is lane-linear;
 //   * the matrix cores compute the tile transposed (D[n][m]) so that each lane
 //     ends up with 4 consecutive n per accumulator quad; a v_permlane32_swap
-//     pairs lanes l / l+32 into 16 consecutive n, scaled, rounded to bf16 and
-//     stored as two 16-byte writes per 32x32 tile;
+//     pairs lanes l / l+32 into 16 consecutive n.  The scaled, bf16-rounded
+//     C tile is staged through the (by then idle) LDS ring and leaves as
+//     whole rows, 1 KiB of consecutive bytes per wave store;
 //   * workgroup -> tile mapping is XCD-aware: the 8 XCDs each get a contiguous
 //     range of a grouped (GROUP_M tall) tile order so that the workgroups
 //     resident on one XCD share A and B panels in that XCD's L2.
