@@ -115,7 +115,7 @@ int l8_gemm_nt(const void *A, const void *B, int64_t M, int64_t N, int64_t K,
  *   h        bf16 [R,C] (ldh) or NULL when the caller does not need the product itself
  *   q, scale, amax, col_amax, workspace: as l8_cast_rowwise; the workspace needs
  *            l8_swiglu_workspace(R, C) / 2 bytes.
- * Requires C % 8 == 0, C <= 32768, every leading dimension % 8 == 0. */
+ * Requires C % 8 == 0, C <= 65536, every leading dimension % 8 == 0. */
 int l8_swiglu_cast_rowwise(const void *h1, const void *h3, int64_t R, int64_t C, int64_t ld1, int64_t ld3,
                            void *h, int64_t ldh, void *q, int64_t ldq, float *scale, void *amax,
                            float *col_amax, void *workspace, int64_t workspace_bytes, void *stream);
@@ -129,7 +129,7 @@ int64_t l8_swiglu_workspace(int64_t R, int64_t C);
  *   then q1 / scale1 and q3 / scale3 as l8_cast_rowwise of g1 and g3.
  *   dh, h1, h3 bf16 [R,C];  g1, g3 bf16 [R,C] (ldg) are always written (wgrad needs them);
  *   col_amax1, col_amax3 fp32 [C]: both or neither; workspace of l8_swiglu_workspace(R, C) bytes with them.
- * Requires C % 8 == 0, C <= 16384, every leading dimension % 8 == 0. */
+ * Requires C % 8 == 0, C <= 32768, every leading dimension % 8 == 0. */
 int l8_swiglu_bwd_cast_rowwise(const void *dh, const void *h1, const void *h3, int64_t R, int64_t C,
                                int64_t lddh, int64_t ld1, int64_t ld3, void *g1, void *g3, int64_t ldg,
                                void *q1, void *q3, int64_t ldq, float *scale1, float *scale3,

@@ -266,14 +266,226 @@ __global__ __launch_bounds__(kGateBlock, 2) void swiglu_bwd_cast_rowwise_kernel(
   }
 }
 
+// Wide rows (ffn dimensions beyond what a 256-thread workgroup holds in
+// registers without spilling): 1024 threads per row, two passes.  Pass 1
+// computes the gate, stores the bf16 result and reduces the row amax; pass 2
+// reads the thread's own bf16 values back (they are still in L2) and casts.
+// Column maxima live in LDS (one bf16 per column and tensor, each owned by one
+// thread).  Any C that is a multiple of 8.
+constexpr int kWideBlock = 1024;
+constexpr int kWideWaves = kWideBlock / 64;
+
+template <bool COLMAX>
+__global__ __launch_bounds__(kWideBlock) void swiglu_cast_rowwise_wide_kernel(
+    const uint16_t *__restrict__ h1, const uint16_t *__restrict__ h3, int64_t R, int C, int64_t ld1, int64_t ld3,
+    uint16_t *__restrict__ hout, int64_t ldh, uint8_t *__restrict__ q, int64_t ldq, float *__restrict__ scale,
+    uint16_t *__restrict__ amax_out, uint16_t *__restrict__ col_partials) {
+  __shared__ uint32_t red[2][kWideWaves];
+  extern __shared__ __attribute__((aligned(16))) uint8_t dyn_lds[];
+  v4i *lds_cm = (v4i *)dyn_lds;  // [C / 8]
+  const int lane = threadIdx.x & 63;
+  const int wave = threadIdx.x >> 6;
+  if (COLMAX)
+    for (int c = threadIdx.x * 8; c < C; c += kWideBlock * 8) lds_cm[c / 8] = v4i{0, 0, 0, 0};
+  int it = 0;
+  for (int64_t r = blockIdx.x; r < R; r += gridDim.x, ++it) {
+    uint32_t m = 0;
+    for (int c = threadIdx.x * 8; c < C; c += kWideBlock * 8) {
+      const v4i a = __builtin_nontemporal_load((const v4i *)(h1 + r * ld1 + c));
+      const v4i b = __builtin_nontemporal_load((const v4i *)(h3 + r * ld3 + c));
+      v4i h;
+#pragma unroll
+      for (int k = 0; k < 4; ++k) {
+        h[k] = (int)gate_fwd2((uint32_t)a[k], (uint32_t)b[k]);
+        m = pk_absmax_u16(m, (uint32_t)h[k]);
+      }
+      if (COLMAX) {
+        v4i old = lds_cm[c / 8];
+#pragma unroll
+        for (int k = 0; k < 4; ++k) old[k] = (int)pk_absmax_u16((uint32_t)old[k], (uint32_t)h[k]);
+        lds_cm[c / 8] = old;
+      }
+      if (hout) *(v4i *)(hout + r * ldh + c) = h;
+    }
+    m = wave_max_u32(max(m & 0xffffu, m >> 16));
+    if (lane == 0) red[it & 1][wave] = m;
+    __syncthreads();
+    uint32_t amax_bits = 0;
+#pragma unroll
+    for (int w = 0; w < kWideWaves; ++w) amax_bits = max(amax_bits, red[it & 1][w]);
+    const RowScale rs = row_scale(amax_bits);
+    if (threadIdx.x == 0) {
+      if (scale) scale[r] = rs.s;
+      if (amax_out) amax_out[r] = (uint16_t)amax_bits;
+    }
+    if (q) {
+      uint8_t *qrow = q + r * ldq;
+      for (int c = threadIdx.x * 8; c < C; c += kWideBlock * 8) {
+        v4i h;
+        if (hout) {
+          h = *(const v4i *)(hout + r * ldh + c);  // this thread's own store of pass 1
+        } else {
+          const v4i a = *(const v4i *)(h1 + r * ld1 + c);
+          const v4i b = *(const v4i *)(h3 + r * ld3 + c);
+#pragma unroll
+          for (int k = 0; k < 4; ++k) h[k] = (int)gate_fwd2((uint32_t)a[k], (uint32_t)b[k]);
+        }
+        if (rs.finite) __builtin_nontemporal_store(cvt8(h, rs.recip), (v2i *)(qrow + c));
+        else *(v2i *)(qrow + c) = cvt8_slow(h, rs.recip);
+      }
+    }
+  }
+  if (COLMAX)
+    for (int c = threadIdx.x * 8; c < C; c += kWideBlock * 8)
+      *(v4i *)(col_partials + (int64_t)blockIdx.x * C + c) = lds_cm[c / 8];
+}
+
+template <bool COLMAX>
+__global__ __launch_bounds__(kWideBlock) void swiglu_bwd_cast_rowwise_wide_kernel(
+    const uint16_t *__restrict__ dh, const uint16_t *__restrict__ h1, const uint16_t *__restrict__ h3, int64_t R, int C,
+    int64_t lddh, int64_t ld1, int64_t ld3, uint16_t *__restrict__ g1out, uint16_t *__restrict__ g3out, int64_t ldg,
+    uint8_t *__restrict__ q1, uint8_t *__restrict__ q3, int64_t ldq, float *__restrict__ scale1,
+    float *__restrict__ scale3, uint16_t *__restrict__ col_partials1, uint16_t *__restrict__ col_partials3) {
+  __shared__ uint32_t red[2][2][kWideWaves];
+  extern __shared__ __attribute__((aligned(16))) uint8_t dyn_lds[];
+  v4i *lds_cm1 = (v4i *)dyn_lds, *lds_cm3 = lds_cm1 + C / 8;  // [C / 8] each
+  const int lane = threadIdx.x & 63;
+  const int wave = threadIdx.x >> 6;
+  if (COLMAX)
+    for (int c = threadIdx.x * 8; c < C; c += kWideBlock * 8) lds_cm1[c / 8] = lds_cm3[c / 8] = v4i{0, 0, 0, 0};
+  int it = 0;
+  for (int64_t r = blockIdx.x; r < R; r += gridDim.x, ++it) {
+    uint32_t m1 = 0, m3 = 0;
+    for (int c = threadIdx.x * 8; c < C; c += kWideBlock * 8) {
+      const v4i d = __builtin_nontemporal_load((const v4i *)(dh + r * lddh + c));
+      const v4i a = __builtin_nontemporal_load((const v4i *)(h1 + r * ld1 + c));
+      const v4i b = __builtin_nontemporal_load((const v4i *)(h3 + r * ld3 + c));
+      v4i g1, g3;
+#pragma unroll
+      for (int k = 0; k < 4; ++k) {
+        uint32_t x1, x3;
+        gate_bwd2((uint32_t)d[k], (uint32_t)a[k], (uint32_t)b[k], x1, x3);
+        g1[k] = (int)x1;
+        g3[k] = (int)x3;
+        m1 = pk_absmax_u16(m1, x1);
+        m3 = pk_absmax_u16(m3, x3);
+      }
+      if (COLMAX) {
+        v4i o1 = lds_cm1[c / 8], o3 = lds_cm3[c / 8];
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+          o1[k] = (int)pk_absmax_u16((uint32_t)o1[k], (uint32_t)g1[k]);
+          o3[k] = (int)pk_absmax_u16((uint32_t)o3[k], (uint32_t)g3[k]);
+        }
+        lds_cm1[c / 8] = o1;
+        lds_cm3[c / 8] = o3;
+      }
+      *(v4i *)(g1out + r * ldg + c) = g1;
+      *(v4i *)(g3out + r * ldg + c) = g3;
+    }
+    m1 = wave_max_u32(max(m1 & 0xffffu, m1 >> 16));
+    m3 = wave_max_u32(max(m3 & 0xffffu, m3 >> 16));
+    if (lane == 0) {
+      red[it & 1][0][wave] = m1;
+      red[it & 1][1][wave] = m3;
+    }
+    __syncthreads();
+    uint32_t bits1 = 0, bits3 = 0;
+#pragma unroll
+    for (int w = 0; w < kWideWaves; ++w) {
+      bits1 = max(bits1, red[it & 1][0][w]);
+      bits3 = max(bits3, red[it & 1][1][w]);
+    }
+    const RowScale rs1 = row_scale(bits1), rs3 = row_scale(bits3);
+    if (threadIdx.x == 0) {
+      scale1[r] = rs1.s;
+      scale3[r] = rs3.s;
+    }
+    uint8_t *q1row = q1 + r * ldq, *q3row = q3 + r * ldq;
+    for (int c = threadIdx.x * 8; c < C; c += kWideBlock * 8) {
+      const v4i g1 = *(const v4i *)(g1out + r * ldg + c);  // this thread's own stores of pass 1
+      const v4i g3 = *(const v4i *)(g3out + r * ldg + c);
+      if (rs1.finite) __builtin_nontemporal_store(cvt8(g1, rs1.recip), (v2i *)(q1row + c));
+      else *(v2i *)(q1row + c) = cvt8_slow(g1, rs1.recip);
+      if (rs3.finite) __builtin_nontemporal_store(cvt8(g3, rs3.recip), (v2i *)(q3row + c));
+      else *(v2i *)(q3row + c) = cvt8_slow(g3, rs3.recip);
+    }
+  }
+  if (COLMAX)
+    for (int c = threadIdx.x * 8; c < C; c += kWideBlock * 8) {
+      *(v4i *)(col_partials1 + (int64_t)blockIdx.x * C + c) = lds_cm1[c / 8];
+      *(v4i *)(col_partials3 + (int64_t)blockIdx.x * C + c) = lds_cm3[c / 8];
+    }
+}
+
 // workgroups (= rows of a partial-maxima array) for R rows
 static int64_t gate_blocks(int64_t R) {
   const int64_t cap = (int64_t)num_cus() * 2;
   return R < cap ? R : cap;
 }
 
-constexpr int64_t kGateMaxC = 16 * kGateWaves * 512;     // forward: 16 chunks per lane
-constexpr int64_t kGateBwdMaxC = 8 * kGateWaves * 512;   // backward keeps two rows in registers
+// the column maxima of the wide kernels must fit LDS: 2 B (forward) or 4 B (backward) per column
+constexpr int64_t kGateMaxC = 65536;
+constexpr int64_t kGateBwdMaxC = 32768;
+
+// dynamic LDS above the default limit needs the attribute once per device
+template <typename K>
+static int allow_lds(K kernel, size_t bytes, bool (&done)[kMaxDev]) {
+  if (bytes <= 48 * 1024) return L8_OK;
+  const int slot = device_slot();
+  if (slot >= 0 && done[slot]) return L8_OK;
+  L8_HIP(hipFuncSetAttribute((const void *)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, 159 * 1024));
+  if (slot >= 0) done[slot] = true;
+  return L8_OK;
+}
+
+static int launch_fwd_wide(const void *h1, const void *h3, int64_t R, int64_t C, int64_t ld1, int64_t ld3, void *h,
+                           int64_t ldh, void *q, int64_t ldq, float *scale, void *amax, float *col_amax, void *ws,
+                           hipStream_t st) {
+  const int64_t blocks = gate_blocks(R);
+  if (col_amax) {
+    static bool done[kMaxDev] = {};
+    const size_t lds = (size_t)C * 2;
+    const int rc = allow_lds(swiglu_cast_rowwise_wide_kernel<true>, lds, done);
+    if (rc != L8_OK) return rc;
+    hipLaunchKernelGGL((swiglu_cast_rowwise_wide_kernel<true>), dim3((unsigned)blocks), dim3(kWideBlock), lds, st,
+                       (const uint16_t *)h1, (const uint16_t *)h3, R, (int)C, ld1, ld3, (uint16_t *)h, ldh, (uint8_t *)q, ldq,
+                       scale, (uint16_t *)amax, (uint16_t *)ws);
+    L8_HIP(hipGetLastError());
+    return fold_colmax(ws, blocks, C, col_amax, st);
+  }
+  hipLaunchKernelGGL((swiglu_cast_rowwise_wide_kernel<false>), dim3((unsigned)blocks), dim3(kWideBlock), 0, st,
+                     (const uint16_t *)h1, (const uint16_t *)h3, R, (int)C, ld1, ld3, (uint16_t *)h, ldh, (uint8_t *)q, ldq,
+                     scale, (uint16_t *)amax, (uint16_t *)nullptr);
+  L8_HIP(hipGetLastError());
+  return L8_OK;
+}
+
+static int launch_bwd_wide(const void *dh, const void *h1, const void *h3, int64_t R, int64_t C, int64_t lddh, int64_t ld1,
+                           int64_t ld3, void *g1, void *g3, int64_t ldg, void *q1, void *q3, int64_t ldq, float *s1,
+                           float *s3, float *ca1, float *ca3, void *ws, hipStream_t st) {
+  const int64_t blocks = gate_blocks(R);
+  if (ca1) {
+    static bool done[kMaxDev] = {};
+    uint16_t *w1 = (uint16_t *)ws, *w3 = w1 + blocks * C;
+    const size_t lds = (size_t)C * 4;
+    int rc = allow_lds(swiglu_bwd_cast_rowwise_wide_kernel<true>, lds, done);
+    if (rc != L8_OK) return rc;
+    hipLaunchKernelGGL((swiglu_bwd_cast_rowwise_wide_kernel<true>), dim3((unsigned)blocks), dim3(kWideBlock), lds, st,
+                       (const uint16_t *)dh, (const uint16_t *)h1, (const uint16_t *)h3, R, (int)C, lddh, ld1, ld3,
+                       (uint16_t *)g1, (uint16_t *)g3, ldg, (uint8_t *)q1, (uint8_t *)q3, ldq, s1, s3, w1, w3);
+    L8_HIP(hipGetLastError());
+    rc = fold_colmax(w1, blocks, C, ca1, st);
+    if (rc != L8_OK) return rc;
+    return fold_colmax(w3, blocks, C, ca3, st);
+  }
+  hipLaunchKernelGGL((swiglu_bwd_cast_rowwise_wide_kernel<false>), dim3((unsigned)blocks), dim3(kWideBlock), 0, st,
+                     (const uint16_t *)dh, (const uint16_t *)h1, (const uint16_t *)h3, R, (int)C, lddh, ld1, ld3,
+                     (uint16_t *)g1, (uint16_t *)g3, ldg, (uint8_t *)q1, (uint8_t *)q3, ldq, s1, s3, (uint16_t *)nullptr,
+                     (uint16_t *)nullptr);
+  L8_HIP(hipGetLastError());
+  return L8_OK;
+}
 
 template <int NCHW>
 static int launch_fwd(const void *h1, const void *h3, int64_t R, int64_t C, int64_t ld1, int64_t ld3, void *h, int64_t ldh,
@@ -370,8 +582,8 @@ extern "C" int l8_swiglu_cast_rowwise(const void *h1, const void *h3, int64_t R,
   if (nchw <= 4) L8_FWD(4);
   if (nchw <= 6) L8_FWD(6);
   if (nchw <= 8) L8_FWD(8);
-  L8_FWD(16);
 #undef L8_FWD
+  return launch_fwd_wide(h1, h3, R, C, ld1, ld3, h, ldh, q, ldq, scale, amax, col_amax, workspace, st);
 }
 
 extern "C" int l8_swiglu_bwd_cast_rowwise(const void *dh, const void *h1, const void *h3, int64_t R, int64_t C, int64_t lddh,
@@ -403,6 +615,7 @@ extern "C" int l8_swiglu_bwd_cast_rowwise(const void *dh, const void *h1, const 
   if (nchw <= 2) L8_BWD(2);
   if (nchw <= 4) L8_BWD(4);
   if (nchw <= 6) L8_BWD(6);
-  L8_BWD(8);
 #undef L8_BWD
+  return launch_bwd_wide(dh, h1, h3, R, C, lddh, ld1, ld3, g1, g3, ldg, q1, q3, ldq, scale1, scale3, col_amax1, col_amax3,
+                         workspace, st);
 }
