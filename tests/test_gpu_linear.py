@@ -358,3 +358,28 @@ def test_empty_batch_and_single_token():
     assert rel_l2(x1.grad, oracle.linear_dgrad(g1.cpu(), W)) <= TOL
     assert rel_l2(lin.weight.grad, oracle.linear_wgrad_fp8(g1.cpu(), x1.detach().cpu())) <= TOL
     assert torch.equal(lin.bias.grad, g1[0])
+
+
+def test_mlp_step_is_bitwise_reproducible():
+    """No result of the path depends on scheduling: the column amaxes are max-merged (order-free), every sum runs
+    in a fixed order.  Two runs of the same MLP step give identical bits, drop-in and fused."""
+    from lingua_amd import convert_linears_to_fp8
+    from lingua_amd.callers import FeedForward
+    from lingua_amd.swiglu import Fp8FeedForward
+    torch.manual_seed(12)
+    holder = nn.ModuleDict({"feed_forward": FeedForward(512, 1536).to(device="cuda", dtype=torch.bfloat16)})
+    mlp = convert_linears_to_fp8(holder, "rowwise", r"feed_forward\.")["feed_forward"]
+    fused = Fp8FeedForward(mlp.w1, mlp.w3, mlp.w2)
+    x = seeded_bf16((1000, 512), seed=51).cuda()
+    gy = seeded_bf16((1000, 512), std=0.02, seed=52).cuda()
+    for module in (mlp, fused):
+        runs = []
+        for _ in range(2):
+            for p in module.parameters():
+                p.grad = None
+            xi = x.clone().requires_grad_(True)
+            y = module(xi)
+            y.backward(gy)
+            runs.append([y.detach(), xi.grad] + [p.grad.clone() for p in module.parameters()])
+        for a, b in zip(*runs):
+            assert torch.equal(a.view(torch.int16), b.view(torch.int16))
