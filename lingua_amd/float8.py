@@ -62,21 +62,47 @@ class Fp8Config:
 config = Fp8Config()
 
 
+def _col_groups(t: torch.Tensor, amax_t: torch.Tensor) -> int:
+    """Number of column groups an amax of shape [R or 1, g] asks for, after checking that the tiling is one
+    the kernels serve: whole rows or the whole tensor in the row direction, g equal groups of a multiple of
+    16 columns in the other (lingua/float8.py:24-30 divides the operand into amax.shape chunks)."""
+    if amax_t.dim() != 2 or amax_t.shape[0] not in (1, t.shape[0]) or amax_t.shape[1] < 1:
+        raise RuntimeError(f"scale: unsupported amax shape {tuple(amax_t.shape)} for input {tuple(t.shape)}")
+    g = amax_t.shape[1]
+    if g > 1 and (t.shape[1] % g or (t.shape[1] // g) % 16):
+        raise RuntimeError(f"scale: {t.shape[1]} columns do not split into {g} groups of a multiple of 16")
+    return g
+
+
 def scale(t: torch.Tensor, amax_t: Optional[torch.Tensor] = None):
     """Quantise ``t`` [R,C] bf16: returns ``(t_fp8, scale_t)`` like lingua/float8.py:43-47.
 
     ``amax_t`` selects the granularity by its shape, as the reference's tile
     broadcast does (lingua/float8.py:24-30): ``[R,1]`` (or None) is row-wise,
-    ``[1,1]`` tensor-wise.  For the row-wise case the amax is recomputed inside
-    the fused kernel (it is a by-product of the same pass), so the values of a
-    given ``[R,1]`` tensor are not read.
+    ``[1,1]`` tensor-wise, ``[R,g]`` sub-row-wise -- every row in ``g`` equal
+    column groups, each with a scale of its own, which is what the reference
+    computes when tensor parallelism shards the reduction dimension over ``g``
+    ranks (lingua/float8.py:14-21, :86).  For the row-wise and sub-row-wise
+    cases the amax is recomputed inside the fused kernel (it is a by-product of
+    the same pass), so the values of the given tensor are not read.
     """
-    if amax_t is None or (amax_t.dim() == 2 and amax_t.shape[0] == t.shape[0] and amax_t.shape[1] == 1 and t.shape[0] != 1):
+    if amax_t is None:
         q, s, _ = ops.cast_rowwise(t)
         return q, s
-    if amax_t.numel() == 1:
-        return ops.cast_tensorwise(t, amax_t.to(torch.bfloat16), transpose=False)
-    raise RuntimeError(f"scale: unsupported amax shape {tuple(amax_t.shape)} for input {tuple(t.shape)}")
+    g = _col_groups(t, amax_t)
+    if g > 1:
+        if amax_t.shape[0] != t.shape[0]:
+            raise RuntimeError(f"scale: unsupported amax shape {tuple(amax_t.shape)} for input {tuple(t.shape)}")
+        cs = t.shape[1] // g
+        q = torch.empty(t.shape, dtype=torch.float8_e4m3fn, device=t.device)
+        s = torch.empty((t.shape[0], g), dtype=torch.float32, device=t.device)
+        for j in range(g):
+            ops.cast_rowwise(t[:, j * cs:(j + 1) * cs], out_q=q[:, j * cs:(j + 1) * cs], out_scale=s[:, j:j + 1])
+        return q, s
+    if amax_t.shape[0] == t.shape[0] and t.shape[0] != 1:
+        q, s, _ = ops.cast_rowwise(t)
+        return q, s
+    return ops.cast_tensorwise(t, amax_t.to(torch.bfloat16), transpose=False)
 
 
 def matmul(first, amax_first, second_t, amax_second_t, bias, use_fast_accum: bool = True):
@@ -84,11 +110,30 @@ def matmul(first, amax_first, second_t, amax_second_t, bias, use_fast_accum: boo
 
     ``use_fast_accum`` is accepted for signature parity; accumulation is always
     fp32 on the matrix cores and the scales are always applied in the epilogue.
+
+    With sub-row-wise amaxes (``[R,g]`` and ``[N,g]``) the product is the sum of
+    ``g`` partial products, one per column group with that group's scales, each
+    rounded to bf16 as the per-rank ``_scaled_mm`` of the reference's
+    tensor-parallel case is (lingua/float8.py:65-77 under a Shard(1) placement);
+    the partials are then added in fp32 and rounded once, where the reference
+    leaves the order of that sum to the all-reduce.
     """
     del use_fast_accum
     q1, s1 = scale(first, amax_first)
     q2, s2 = scale(second_t, amax_second_t)
-    return ops.gemm_nt(q1, q2, s1, s2, bias, algo=config.gemm_algo)
+    g1 = s1.shape[1] if s1.dim() == 2 else 1
+    g2 = s2.shape[1] if s2.dim() == 2 else 1
+    if g1 == 1 and g2 == 1:
+        return ops.gemm_nt(q1, q2, s1, s2, bias, algo=config.gemm_algo)
+    if g1 != g2:
+        raise RuntimeError(f"matmul: operands are scaled in {g1} and {g2} column groups")
+    cs = q1.shape[1] // g1
+    acc = None
+    for j in range(g1):
+        part = ops.gemm_nt(q1[:, j * cs:(j + 1) * cs], q2[:, j * cs:(j + 1) * cs], s1[:, j], s2[:, j],
+                           bias if j == 0 else None, algo=config.gemm_algo)
+        acc = part.float() if acc is None else acc.add_(part)
+    return acc.to(torch.bfloat16)
 
 
 class _LastCast:

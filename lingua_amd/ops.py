@@ -59,14 +59,21 @@ def _ld(t: torch.Tensor) -> int:
     return t.stride(0) if t.shape[0] > 1 else max(t.shape[1], 1)
 
 
-def cast_rowwise(x: torch.Tensor, col_amax: Optional[torch.Tensor] = None, want_q: bool = True):
+def cast_rowwise(x: torch.Tensor, col_amax: Optional[torch.Tensor] = None, want_q: bool = True,
+                 out_q: Optional[torch.Tensor] = None, out_scale: Optional[torch.Tensor] = None):
     """Row-wise amax -> scale -> e4m3fn.  Returns (q [R,C] fp8 | None, scale [R,1] fp32, amax [R,1] bf16).
 
-    ``col_amax`` (fp32 [C], zero-initialised by the caller) is max-merged with the column amaxes of x."""
+    ``col_amax`` (fp32 [C], zero-initialised by the caller) is max-merged with the column amaxes of x.
+    ``out_q`` (fp8 [R,C], unit column stride, row stride a multiple of 8) and ``out_scale`` (fp32 [R,1], any
+    strides) receive the results in place of fresh tensors: a column slice of a wider matrix is the use."""
     x = _rows_2d(x, torch.bfloat16, "cast_rowwise")
     st = _prep(x, "cast_rowwise")
     R, C = x.shape
-    q = torch.empty((R, C), dtype=torch.float8_e4m3fn, device=x.device) if want_q else None
+    q = None
+    if want_q:
+        q = out_q if out_q is not None else torch.empty((R, C), dtype=torch.float8_e4m3fn, device=x.device)
+        if q.dtype != torch.float8_e4m3fn or tuple(q.shape) != (R, C) or q.device != x.device or (q.numel() and q.stride(1) != 1):
+            raise RuntimeError("cast_rowwise: out_q must be an e4m3fn [R,C] tensor on x's device with unit column stride")
     scale = torch.empty((R, 1), dtype=torch.float32, device=x.device)
     amax = torch.empty((R, 1), dtype=torch.bfloat16, device=x.device)
     if col_amax is not None and (col_amax.dtype != torch.float32 or col_amax.numel() != C or not col_amax.is_contiguous()):
@@ -78,10 +85,14 @@ def cast_rowwise(x: torch.Tensor, col_amax: Optional[torch.Tensor] = None, want_
             ws = torch.empty(ws_bytes, dtype=torch.uint8, device=x.device)
     with _timed("cast_rowwise", R * C * (3 if want_q else 2) + 4 * R + (4 * C if col_amax is not None else 0), x.device):
         code = _lib.load().l8_cast_rowwise(
-            x.data_ptr(), R, C, _ld(x), q.data_ptr() if want_q else None, C, scale.data_ptr(), amax.data_ptr(),
-            col_amax.data_ptr() if col_amax is not None else None, ws.data_ptr() if ws is not None else None,
-            ws_bytes, st)
+            x.data_ptr(), R, C, _ld(x), q.data_ptr() if want_q else None, _ld(q) if want_q else C, scale.data_ptr(),
+            amax.data_ptr(), col_amax.data_ptr() if col_amax is not None else None,
+            ws.data_ptr() if ws is not None else None, ws_bytes, st)
     _lib.check(code, "l8_cast_rowwise")
+    if out_scale is not None:
+        if out_scale.dtype != torch.float32 or tuple(out_scale.shape) != (R, 1):
+            raise RuntimeError("cast_rowwise: out_scale must be fp32 [R,1]")
+        scale = out_scale.copy_(scale)
     return q, scale, amax
 
 

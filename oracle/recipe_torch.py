@@ -26,21 +26,44 @@ def tensor_amax_from_rows(amax_rows: torch.Tensor, n_rows_out: int) -> torch.Ten
     return a.repeat_interleave(n_rows_out // a.shape[0], dim=0, output_size=n_rows_out)
 
 
+def tile_broadcast(b: torch.Tensor, shape) -> torch.Tensor:
+    """lingua/float8.py:24-30 as an expansion: b [m,n] -> [R,C] where element (r,c) is b[r // (R/m), c // (C/n)],
+    i.e. the operand is cut into m x n equal chunks and each chunk sees one element of b."""
+    R, C = shape
+    m, n = b.shape
+    return b.repeat_interleave(R // m, dim=0).repeat_interleave(C // n, dim=1)
+
+
 def scale(t: torch.Tensor, amax_t: torch.Tensor):
-    """lingua/float8.py:43-47.  amax_t is [R,1] (row-wise) or [1,1] (tensor-wise)."""
+    """lingua/float8.py:43-47.  amax_t is [R,1] (row-wise), [1,1] (tensor-wise) or [R,g] (g column groups per row)."""
     scale_t = torch.clamp(amax_t.float(), min=EPS) / E4M3_MAX
     recip = scale_t.reciprocal()
-    # tile broadcast of lingua/float8.py:24-30 for [R,1] and [1,1] scales
-    t_fp8 = (t * recip).to(torch.float8_e4m3fn)
+    t_fp8 = (t * tile_broadcast(recip, t.shape)).to(torch.float8_e4m3fn)
     return t_fp8, scale_t
 
 
+def subrow_amax(t: torch.Tensor, g: int) -> torch.Tensor:
+    """lingua/float8.py:86 with splitk == g: [R,C] -> [R,g] amax of each of the g column groups of a row."""
+    return t.abs().unflatten(-1, (g, -1)).amax(dim=-1)
+
+
 def dequant_matmul(q1, s1, q2_t, s2_t, bias=None) -> torch.Tensor:
-    """bf16( (q1*s1) @ (q2_t*s2_t)^T + bias ), fp32 throughout."""
-    res = (q1.float() * s1) @ (q2_t.float() * s2_t).t()
-    if bias is not None:
-        res = res + bias.float()
-    return res.to(torch.bfloat16)
+    """bf16( (q1*s1) @ (q2_t*s2_t)^T + bias ), fp32 throughout.  With g > 1 scale columns the result is the
+    fp32 sum of the g per-group products, each rounded to bf16 first (one rank's output under tensor
+    parallelism, lingua/float8.py:14-21 and :65-77), rounded to bf16 once more."""
+    g = s1.shape[1]
+    if g == 1 and s2_t.shape[1] == 1:
+        res = (q1.float() * s1) @ (q2_t.float() * s2_t).t()
+        if bias is not None:
+            res = res + bias.float()
+        return res.to(torch.bfloat16)
+    assert s2_t.shape[1] == g
+    cs = q1.shape[1] // g
+    acc = torch.zeros((q1.shape[0], q2_t.shape[0]), dtype=torch.float32)
+    for j in range(g):
+        sl = slice(j * cs, (j + 1) * cs)
+        acc += dequant_matmul(q1[:, sl], s1[:, j:j + 1], q2_t[:, sl], s2_t[:, j:j + 1], bias if j == 0 else None).float()
+    return acc.to(torch.bfloat16)
 
 
 def matmul(first, amax_first, second_t, amax_second_t, bias=None) -> torch.Tensor:

@@ -1,0 +1,67 @@
+"""GPU parity of sub-row-wise scaling: amax of shape [R,g], the granularity the reference uses when tensor
+parallelism shards the reduction dimension over g ranks (lingua/float8.py:14-21, :24-30, :86).  On one GPU
+scale() and matmul() serve it group by group on the row-wise kernels; e4m3 bytes and scales are bit-exact
+against the oracle, the product within rel-L2 1e-3 of the oracle's sum of bf16 partial products."""
+import pytest
+import torch
+
+import oracle
+from oracle import recipe_torch as rt
+from conftest import rel_l2, seeded_bf16
+from golden_util import bits_equal
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.mark.parametrize("shape,g", [((6, 96), 2), ((6, 96), 3), ((1, 64), 4), ((300, 1024), 8), ((65, 4096), 2)])
+def test_scale_with_column_groups(shape, g):
+    from lingua_amd import float8 as f8
+    x = seeded_bf16(shape, std=2.0, seed=shape[0] + g)
+    x[0, : shape[1] // g] = 0.0                    # one all-zero group: scale floor in that group only
+    x[-1, shape[1] - 1] = 200.0                    # an outlier confined to the last group
+    amax = rt.subrow_amax(x, g)
+    q, s = f8.scale(x.cuda(), amax.cuda())
+    want_q, want_s = rt.scale(x, amax)
+    assert q.shape == x.shape and s.shape == (shape[0], g) and s.dtype == torch.float32
+    assert torch.equal(q.cpu().view(torch.uint8), want_q.view(torch.uint8))
+    assert bits_equal(s.cpu(), want_s)
+    assert s.cpu().view(torch.int32)[0, 0].item() == 0x2720D7C5
+    # finer groups never quantise worse than whole rows
+    qr, sr = f8.scale(x.cuda(), rt.row_amax(x).cuda())
+    deq = lambda qq, ss: qq.cpu().float() * rt.tile_broadcast(ss.cpu(), x.shape)
+    assert rel_l2(deq(q, s), x.float()) <= rel_l2(deq(qr, sr), x.float()) * 1.02
+
+
+@pytest.mark.parametrize("mkn,g", [((40, 96, 24), 2), ((130, 1024, 200), 4), ((257, 2048, 513), 8)])
+@pytest.mark.parametrize("with_bias", [False, True])
+def test_matmul_with_column_groups(mkn, g, with_bias):
+    from lingua_amd import float8 as f8
+    M, K, N = mkn
+    a = seeded_bf16((M, K), std=1.5, seed=M)
+    b_t = seeded_bf16((N, K), std=0.05, seed=N)
+    a[3, K // g: 2 * K // g] *= 50.0
+    bias = seeded_bf16((N,), std=0.5, seed=7) if with_bias else None
+    am_a, am_b = rt.subrow_amax(a, g), rt.subrow_amax(b_t, g)
+    got = f8.matmul(a.cuda(), am_a.cuda(), b_t.cuda(), am_b.cuda(), bias.cuda() if with_bias else None)
+    want = rt.matmul(a, am_a, b_t, am_b, bias)
+    assert got.dtype == torch.bfloat16 and got.shape == (M, N)
+    assert rel_l2(got, want) <= 1e-3, rel_l2(got, want)
+    # and it is a better product than whole-row scaling when a group holds outliers
+    exact = a.double() @ b_t.double().t() + (bias.double() if with_bias else 0.0)
+    rowwise = f8.matmul(a.cuda(), rt.row_amax(a).cuda(), b_t.cuda(), rt.row_amax(b_t).cuda(), bias.cuda() if with_bias else None)
+    assert rel_l2(got.double().cpu(), exact) <= rel_l2(rowwise.double().cpu(), exact) * 1.05
+
+
+def test_rejected_tilings():
+    from lingua_amd import float8 as f8
+    x = seeded_bf16((8, 96)).cuda()
+    with pytest.raises(RuntimeError, match="groups"):
+        f8.scale(x, torch.ones(8, 4, device="cuda"))          # 24 columns per group: not a multiple of 16
+    with pytest.raises(RuntimeError, match="groups"):
+        f8.scale(x, torch.ones(8, 5, device="cuda"))          # does not divide
+    with pytest.raises(RuntimeError, match="unsupported amax shape"):
+        f8.scale(x, torch.ones(4, 1, device="cuda"))          # row blocks other than 1 and R
+    with pytest.raises(RuntimeError, match="unsupported amax shape"):
+        f8.scale(x, torch.ones(1, 2, device="cuda"))
+    with pytest.raises(RuntimeError, match="column groups"):
+        f8.matmul(x, torch.ones(8, 2, device="cuda"), x, torch.ones(8, 3, device="cuda"), None)

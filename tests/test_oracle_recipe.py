@@ -213,3 +213,50 @@ def test_rmsnorm_oracle_against_float64():
     z = torch.full((1, 64), -3.0, dtype=torch.bfloat16)
     assert torch.equal(rt.rmsnorm(z, torch.ones(64, dtype=torch.bfloat16), 1e-6), torch.full((1, 64), -1.0, dtype=torch.bfloat16))
     assert float(rt.rmsnorm(torch.zeros((1, 64), dtype=torch.bfloat16), torch.ones(64), 1e-6).abs().max()) == 0.0
+
+
+def test_tiled_scale_oracle_against_slices_and_a_plain_loop():
+    """The [R,g] branch of the oracle's scale(): (1) every column group must come out as the row-wise C oracle
+    (pinned by the golden vectors) quantises that group on its own; (2) the tile expansion is checked element by
+    element against index arithmetic on a shape where a transposed or row/column-swapped expansion differs;
+    (3) g = 1 and [1,1] reduce to the branches the golden vectors cover."""
+    x = seeded_bf16((6, 96), std=2.0, seed=31)
+    x[2, 32:64] = 0.0
+    x[4, 5] = 300.0
+    for g in (1, 2, 3, 6):
+        amax = rt.subrow_amax(x, g)
+        assert amax.shape == (6, g) and amax.dtype == torch.bfloat16
+        q, s = rt.scale(x, amax)
+        cs = 96 // g
+        for j in range(g):
+            qj, sj, aj = oracle.cast_rowwise(x[:, j * cs:(j + 1) * cs].contiguous())
+            assert torch.equal(q[:, j * cs:(j + 1) * cs].view(torch.uint8), qj), (g, j)
+            assert bits_equal(s[:, j].contiguous(), sj) and bits_equal(amax[:, j].contiguous(), aj)
+    b = torch.arange(6, dtype=torch.float32).reshape(2, 3)
+    e = rt.tile_broadcast(b, (4, 12))
+    for r in range(4):
+        for c in range(12):
+            assert e[r, c] == b[r // 2, c // 4]
+    q1, s1 = rt.scale(x, x.abs().amax().reshape(1, 1))
+    q2, s2 = oracle.cast_tensorwise(x)
+    assert torch.equal(q1.view(torch.uint8), q2) and bits_equal(s1.reshape(-1), s2.reshape(-1))
+
+
+def test_subrow_product_oracle_reduces_to_known_cases():
+    """dequant_matmul with g scale columns: equal to the plain product when all groups share one scale and the
+    values are small integers (every partial and the sum are exact in bf16), and group j's scales must reach
+    group j's columns only (a product with one group zeroed loses exactly that group's term)."""
+    g, cs = 4, 16
+    gen = torch.Generator().manual_seed(5)
+    qa = torch.randint(-2, 3, (5, g * cs), generator=gen).float().to(torch.float8_e4m3fn)
+    qb = torch.randint(-2, 3, (7, g * cs), generator=gen).float().to(torch.float8_e4m3fn)
+    ones_a, ones_b = torch.ones(5, g), torch.ones(7, g)
+    want = (qa.float() @ qb.float().t())
+    assert torch.equal(rt.dequant_matmul(qa, ones_a, qb, ones_b).float(), want)
+    sa = torch.tensor([1.0, 2.0, 4.0, 8.0]).repeat(5, 1)
+    sb = torch.tensor([1.0, 0.5, 0.25, 0.125]).repeat(7, 1)
+    assert torch.equal(rt.dequant_matmul(qa, sa, qb, sb).float(), want)      # sa*sb == 1 in every group
+    sa0 = ones_a.clone()
+    sa0[:, 2] = 0.0
+    lost = qa[:, 2 * cs:3 * cs].float() @ qb[:, 2 * cs:3 * cs].float().t()
+    assert torch.equal(rt.dequant_matmul(qa, sa0, qb, ones_b).float(), want - lost)
