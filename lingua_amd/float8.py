@@ -57,6 +57,11 @@ class Fp8Config:
     # (opaque to torch.compile, nameable in activation-checkpointing policies)
     # instead of the plain autograd.Function
     use_custom_ops: bool = False
+    # with fp8_wgrad: quantise the input along the token dimension already in
+    # forward and keep that e4m3 [K,M] copy (+ K scales) for wgrad instead of the
+    # bf16 input: half the bytes held between forward and backward, the same
+    # kernels and the same results (plain autograd.Function route only)
+    save_fp8_input: bool = False
 
 
 config = Fp8Config()
@@ -167,6 +172,7 @@ class _LastCast:
 
 _fwd_cast = _LastCast()   # a -> (qa, sa, a_col_amax | None)
 _bwd_cast = _LastCast()   # a -> (qat, sat)
+_fwd_tcast = _LastCast()  # a -> (qat, sat), made in forward when config.save_fp8_input
 
 
 def linear_forward(a, b_t, bias, need_wgrad_stats: bool, gemm_algo: int):
@@ -191,14 +197,30 @@ def linear_forward(a, b_t, bias, need_wgrad_stats: bool, gemm_algo: int):
     return out, amax_b_t, a_col_amax
 
 
+def input_cast_for_wgrad(a, a_col_amax, user):
+    """``a`` [M,K] quantised along the token dimension into the [K,M] layout wgrad multiplies with, in forward;
+    linears applied to the same activation share one copy."""
+    hit = _fwd_tcast.get(a, user) if config.share_input_casts else None
+    if hit is not None:
+        return hit
+    value = ops.cast_colwise_transposed(a, a_col_amax)
+    if config.share_input_casts:
+        _fwd_tcast.put(a, value, user)
+    return value
+
+
 def linear_backward(grad_out, a, b_t, amax_b_t, a_col_amax, need_a: bool, need_b: bool, need_bias: bool,
-                    fp8_wgrad: bool, gemm_algo: int):
+                    fp8_wgrad: bool, gemm_algo: int, a_tcast=None):
     """Backward of lingua/float8.py:99-131 (fp8 wgrad optional).  Returns ``(grad_a, grad_b, grad_bias)`` with
-    ``None`` where not needed."""
+    ``None`` where not needed.  ``a_tcast`` = ``(qat [K,M], sat [K,1])`` made in forward stands in for ``a``
+    (then ``a`` may be None; fp8 wgrad only)."""
     if grad_out.dtype != torch.bfloat16:
         raise RuntimeError(f"Fp8LinearFn.backward: bf16 grad_out required, got {grad_out.dtype}")
     fp8_wgrad = fp8_wgrad and need_b
     _fwd_cast.clear()
+    _fwd_tcast.clear()
+    if a is None and need_b and not (fp8_wgrad and a_tcast is not None):
+        raise RuntimeError("Fp8LinearFn.backward: the bf16 input was not saved and no quantised copy stands in for it")
 
     g_col_amax = None
     if need_a:
@@ -217,8 +239,10 @@ def linear_backward(grad_out, a, b_t, amax_b_t, a_col_amax, need_a: bool, need_b
             if g_col_amax is None:
                 g_col_amax = ops.col_amax(grad_out)
             qgt, sgt = ops.cast_colwise_transposed(grad_out, g_col_amax)
-            hit = _bwd_cast.get(a, b_t.data_ptr()) if config.share_input_casts else None
-            if hit is not None:
+            hit = _bwd_cast.get(a, b_t.data_ptr()) if config.share_input_casts and a_tcast is None else None
+            if a_tcast is not None:
+                qat, sat = a_tcast
+            elif hit is not None:
                 qat, sat = hit
             else:
                 if a_col_amax is None:
@@ -248,8 +272,13 @@ class Fp8LinearFn(torch.autograd.Function):
         ctx.bias_requires_grad = bias.requires_grad if bias is not None else False
         ctx.fp8_wgrad = config.fp8_wgrad
         ctx.gemm_algo = config.gemm_algo
-        ctx.has_col_amax = a_col_amax is not None
-        if a_col_amax is not None:
+        ctx.kept = "a"
+        if need_wgrad_stats and config.save_fp8_input:
+            qat, sat = input_cast_for_wgrad(a, a_col_amax, b_t.data_ptr())
+            ctx.kept = "a_tcast"
+            ctx.save_for_backward(b_t, amax_b_t, qat, sat)
+        elif a_col_amax is not None:
+            ctx.kept = "a+col"
             ctx.save_for_backward(a, b_t, amax_b_t, a_col_amax)
         else:
             ctx.save_for_backward(a, b_t, amax_b_t)
@@ -257,13 +286,16 @@ class Fp8LinearFn(torch.autograd.Function):
 
     @staticmethod
     def backward(ctx, grad_out):
-        if ctx.has_col_amax:
+        a = a_col_amax = a_tcast = None
+        if ctx.kept == "a_tcast":
+            b_t, amax_b_t, qat, sat = ctx.saved_tensors
+            a_tcast = (qat, sat)
+        elif ctx.kept == "a+col":
             a, b_t, amax_b_t, a_col_amax = ctx.saved_tensors
         else:
             a, b_t, amax_b_t = ctx.saved_tensors
-            a_col_amax = None
         return linear_backward(grad_out, a, b_t, amax_b_t, a_col_amax, ctx.a_requires_grad, ctx.b_requires_grad,
-                               ctx.bias_requires_grad, ctx.fp8_wgrad, ctx.gemm_algo)
+                               ctx.bias_requires_grad, ctx.fp8_wgrad, ctx.gemm_algo, a_tcast)
 
 
 class Fp8Linear(torch.nn.Linear):

@@ -383,3 +383,53 @@ def test_mlp_step_is_bitwise_reproducible():
             runs.append([y.detach(), xi.grad] + [p.grad.clone() for p in module.parameters()])
         for a, b in zip(*runs):
             assert torch.equal(a.view(torch.int16), b.view(torch.int16))
+
+
+def test_fp8_copy_of_the_input_kept_for_wgrad_instead_of_the_bf16_input():
+    """config.save_fp8_input: forward keeps the input quantised along the token dimension (e4m3 [K,M] + K scales)
+    and not the bf16 input; same kernels on the same data, so every result is bit-identical; two linears on one
+    activation share that copy; the bytes held by the graph between forward and backward drop."""
+    from lingua_amd import Fp8Linear, float8, ops
+    torch.manual_seed(6)
+    l1 = Fp8Linear(512, 1024, bias=True, device="cuda", dtype=torch.bfloat16)
+    l3 = Fp8Linear(512, 256, bias=False, device="cuda", dtype=torch.bfloat16)
+    x = seeded_bf16((3, 100, 512), seed=23).cuda().requires_grad_(True)      # 300 tokens: padded to 304 in the [K,M] copy
+    g1 = seeded_bf16((3, 100, 1024), std=0.02, seed=24).cuda()
+    g3 = seeded_bf16((3, 100, 256), std=0.02, seed=25).cuda()
+
+    def run(lean):
+        old = float8.config.save_fp8_input
+        float8.config.save_fp8_input = lean
+        kept, rec = [], []
+        ops.kernel_timer = rec
+        try:
+            for p in (l1.weight, l1.bias, l3.weight, x):
+                p.grad = None
+            with torch.autograd.graph.saved_tensors_hooks(lambda t: (kept.append((t.dtype, tuple(t.shape))), t)[1], lambda t: t):
+                y1, y3 = l1(x), l3(x)
+            n_t_fwd = sum(1 for r in rec if r[0] == "cast_colwise_t")
+            torch.autograd.backward((y1, y3), (g1, g3))
+            n_t_all = sum(1 for r in rec if r[0] == "cast_colwise_t")
+        finally:
+            ops.kernel_timer = None
+            float8.config.save_fp8_input = old
+        outs = [y1.detach(), y3.detach(), x.grad.clone(), l1.weight.grad.clone(), l1.bias.grad.clone(), l3.weight.grad.clone()]
+        return outs, kept, (n_t_fwd, n_t_all)
+
+    plain, kept_plain, n_plain = run(False)
+    lean, kept_lean, n_lean = run(True)
+    for a, b in zip(lean, plain):
+        assert torch.equal(a.view(torch.int16), b.view(torch.int16))
+    assert (torch.bfloat16, (300, 512)) in kept_plain
+    assert (torch.bfloat16, (300, 512)) not in kept_lean
+    assert kept_lean.count((torch.float8_e4m3fn, (512, 304))) == 2          # one shared copy, saved by both linears
+    assert n_plain == (0, 3) and n_lean == (1, 3)                             # x once (forward) + the two grads
+    # without fp8 wgrad, or when the weight does not learn, there is nothing to keep in fp8
+    old = (float8.config.save_fp8_input, float8.config.fp8_wgrad)
+    float8.config.save_fp8_input, float8.config.fp8_wgrad = True, False
+    try:
+        x.grad = l3.weight.grad = None
+        l3(x).backward(g3)
+        assert rel_l2(l3.weight.grad, plain[5]) < 5e-2
+    finally:
+        float8.config.save_fp8_input, float8.config.fp8_wgrad = old
