@@ -47,6 +47,9 @@ def parse():
     ap.add_argument("--no-extras", action="store_true",
                     help="skip the two side measurements: the fused-SwiGLU variant of the same MLP and "
                          "torch._scaled_mm (what the reference calls) on the step's GEMM shapes")
+    ap.add_argument("--gemm-shape", choices=["fwd", "dgrad", "wgrad"], default="fwd",
+                    help="with --kernel-only gemm: which product of the 4096 -> 11008 linear (reduction 4096, 11008, 16384)")
+    ap.add_argument("--launches", type=int, default=3, help="with --kernel-only gemm: number of launches")
     ap.add_argument("--kernel-only", choices=["gemm", "copy", "casts"], default=None,
                     help="profiling aid: launch only the forward-shape GEMM, or a plain 256 MiB device copy "
                          "(the reference point the FETCH_SIZE / WRITE_SIZE counters are scaled by), or each cast "
@@ -250,17 +253,19 @@ def main():
         print(json.dumps({"kernel_only": "copy", "bytes_read": n, "bytes_written": n, "launches": 3}))
         return
     if args.kernel_only == "gemm":
+        M, N, K = {"fwd": (TOKENS, FFN, DIM), "dgrad": (TOKENS, DIM, FFN), "wgrad": (FFN, DIM, TOKENS)}[args.gemm_shape]
         g = torch.Generator().manual_seed(2)
-        a = torch.randn(TOKENS, DIM, generator=g).to(torch.bfloat16).to(dev)
-        b = (torch.randn(FFN, DIM, generator=g) * 0.02).to(torch.bfloat16).to(dev)
+        a = torch.randn(M, K, generator=g).to(torch.bfloat16).to(dev)
+        b = (torch.randn(N, K, generator=g) * 0.02).to(torch.bfloat16).to(dev)
         qa, sa, _ = ops.cast_rowwise(a)
         qb, sb, _ = ops.cast_rowwise(b)
-        out = torch.empty(TOKENS, FFN, dtype=torch.bfloat16, device=dev)
-        for _ in range(3):
+        out = torch.empty(M, N, dtype=torch.bfloat16, device=dev)
+        for _ in range(args.launches):
             ops.gemm_nt(qa, qb, sa, sb, algo=args.algo, out=out)
         torch.cuda.synchronize()
-        print(json.dumps({"kernel_only": "gemm", "M": TOKENS, "N": FFN, "K": DIM, "launches": 3,
-                          "algorithmic_bytes": TOKENS * DIM + FFN * DIM + 2 * TOKENS * FFN + 4 * (TOKENS + FFN)}))
+        print(json.dumps({"kernel_only": "gemm", "M": M, "N": N, "K": K, "launches": args.launches,
+                          "flop_per_launch": 2 * M * N * K,
+                          "algorithmic_bytes": M * K + N * K + 2 * M * N + 4 * (M + N)}))
         return
 
     if args.kernel_only == "casts":
