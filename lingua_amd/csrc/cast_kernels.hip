@@ -219,12 +219,16 @@ __global__ __launch_bounds__(kRowBlock, (NCHW <= 4 ? 4 : (NCHW <= 8 ? 2 : 1))) v
 }
 
 // Folds the partial column maxima [n_slots, C] (bf16) into col_amax[C] (fp32 bit
-// patterns, max-merged).  Thread (x, y): column pair x, slots y*32 .. y*32+31.
+// patterns, max-merged).  Thread (x, y): column pair x, slots y*kFoldSlots .. +kFoldSlots-1.
+#ifndef L8_FOLD_SLOTS
+#define L8_FOLD_SLOTS 8
+#endif
+constexpr int kFoldSlots = L8_FOLD_SLOTS;
 __global__ __launch_bounds__(256) void colmax_fold_kernel(const uint16_t *__restrict__ partials, int n_slots, int C,
                                                           uint32_t *__restrict__ col_amax) {
   const int pair = blockIdx.x * 256 + threadIdx.x;
   if (pair * 2 >= C) return;
-  const int s0 = blockIdx.y * 32, s1 = (s0 + 32 < n_slots) ? s0 + 32 : n_slots;
+  const int s0 = blockIdx.y * kFoldSlots, s1 = (s0 + kFoldSlots < n_slots) ? s0 + kFoldSlots : n_slots;
   uint32_t m = 0;
   for (int sl = s0; sl < s1; ++sl)
     m = pk_absmax_u16(m, __builtin_nontemporal_load((const uint32_t *)(partials + (int64_t)sl * C) + pair));
@@ -519,8 +523,8 @@ static int64_t rowwise_blocks(int64_t R, int64_t C, bool colmax) {
 }
 
 int fold_colmax(const void *partials, int64_t slots, int64_t C, float *col_amax, hipStream_t st) {
-  hipLaunchKernelGGL(colmax_fold_kernel, dim3((unsigned)((C / 2 + 255) / 256), (unsigned)((slots + 31) / 32)), dim3(256), 0,
-                     st, (const uint16_t *)partials, (int)slots, (int)C, (uint32_t *)col_amax);
+  hipLaunchKernelGGL(colmax_fold_kernel, dim3((unsigned)((C / 2 + 255) / 256), (unsigned)((slots + kFoldSlots - 1) / kFoldSlots)),
+                     dim3(256), 0, st, (const uint16_t *)partials, (int)slots, (int)C, (uint32_t *)col_amax);
   L8_HIP(hipGetLastError());
   return L8_OK;
 }
