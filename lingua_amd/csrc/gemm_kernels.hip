@@ -444,12 +444,14 @@ __global__ __launch_bounds__(WM *WN * 64) void gemm_nt_kernel(const GemmArgs p) 
   static_assert((NW * 64) % CPR == 0, "a wave store covers whole rows");
   const int row0 = (wave * 64 + lane) / CPR, col = ((wave * 64 + lane) % CPR) * 8;
   if (c_vec && m0 + BM <= p.M && n0 + BN <= p.N && L8_GEMM_DIAG != 3) {
-    // interior tile: no masks, one pointer and one LDS address stepped by constants
+    // interior tile: no masks, one pointer and one LDS address stepped by constants; streaming stores, so
+    // that the C tile on its way out does not push the operand panels out of the L2
     uint16_t *dst = p.C + (int64_t)(m0 + row0) * p.ldc + n0 + col;
     const uint32_t at = lds0 + row0 * C_ROW + col * 2;
 #pragma unroll
     for (int it = 0; it < ITERS; ++it)
-      *(v4i *)(dst + (int64_t)it * ROWS_PER_IT * p.ldc) = *reinterpret_cast<lds_v4i_ptr>(at + it * (ROWS_PER_IT * C_ROW));
+      __builtin_nontemporal_store(*reinterpret_cast<lds_v4i_ptr>(at + it * (ROWS_PER_IT * C_ROW)),
+                                  (v4i *)(dst + (int64_t)it * ROWS_PER_IT * p.ldc));
   } else if (L8_GEMM_DIAG != 3) {
 #pragma unroll 4
     for (int it = 0; it < ITERS; ++it) {
@@ -459,7 +461,7 @@ __global__ __launch_bounds__(WM *WN * 64) void gemm_nt_kernel(const GemmArgs p) 
       if (m < p.M && n < p.N) {
         uint16_t *dst = p.C + (int64_t)m * p.ldc + n;
         if (c_vec && n + 8 <= p.N) {
-          *(v4i *)dst = v;
+          __builtin_nontemporal_store(v, (v4i *)dst);
         } else {
 #pragma unroll
           for (int e = 0; e < 8; ++e)
@@ -519,11 +521,12 @@ extern "C" const char *l8_gemm_algo_name(int algo) {
 
 static int pick_algo(int64_t M, int64_t N, int64_t K) {
   // large problems: 256x256 tiles -- four waves with 128x128 wave tiles (least
-  // LDS traffic per flop) when the K loop dominates, eight waves when K is short
-  // and the C tile's trip through LDS and out to memory weighs more; problems
-  // that would leave most of the chip idle with big tiles: 128x128
+  // LDS traffic per flop) unless K is so short (measured: below 4096) that the
+  // conversion of the C tile, which eight waves share out over twice as many
+  // wave slots, weighs more than the K loop; problems that would leave most of
+  // the chip idle with big tiles: 128x128
   const int64_t big_tiles = ((M + 255) / 256) * ((N + 255) / 256);
-  if (big_tiles >= num_cus()) return K >= 8192 ? 5 : 3;
+  if (big_tiles >= num_cus()) return K >= 4096 ? 5 : 3;
   return 2;
 }
 
