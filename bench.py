@@ -26,9 +26,10 @@ DIM, FFN, TOKENS = 4096, 11008, 16384
 STEP_FLOP = 18 * TOKENS * DIM * FFN          # 9 GEMMs x 2*M*N*K
 PEAK_FP8_TFLOPS = 5000.0                     # MI355X dense fp8 MFMA, published
 PEAK_HBM_GBPS = 8000.0                       # MI355X HBM3E, published
-# HBM-side bytes per forward-shape GEMM launch from rocprofv3 FETCH_SIZE / WRITE_SIZE, each scaled by what the
-# same counter reads for a 256 MiB copy (profiles/gemm_nt_7b_fwd_hbm_traffic.txt): 1.126 GB read + 0.440 GB written
-GEMM_TRAFFIC_BYTES = 1_488_000_000
+# HBM-side bytes per GEMM launch from rocprofv3 FETCH_SIZE / WRITE_SIZE, each scaled by what the same counter reads
+# for a 256 MiB copy (profiles/gemm_nt_7b_hbm_traffic.txt), mean over the three products the step launches three
+# times each: forward 1.486 GB, dgrad 1.226 GB, wgrad 1.456 GB (algorithmic: 473 / 360 / 338 MB)
+GEMM_TRAFFIC_BYTES = 1_389_000_000
 
 
 def parse():
@@ -361,10 +362,10 @@ def main():
                                  "frac_hbm": round(gbps / PEAK_HBM_GBPS, 4)}
         n, ms, work = agg["gemm_nt"]
         achieved = work / (ms * 1e-3) / 1e12
-        roofline = {"kernel": "gemm_nt_kernel (fp8 e4m3 NT GEMM, 2*16384*4096*11008 flop per launch)",
+        roofline = {"kernel": "gemm_nt_kernel (fp8 e4m3 NT GEMM, 2*16384*4096*11008 flop per launch; forward, dgrad and wgrad products)",
                     "bound": "mfma", "achieved": round(achieved, 1), "peak": PEAK_FP8_TFLOPS, "unit": "TFLOP/s",
                     "frac": round(achieved / PEAK_FP8_TFLOPS, 4), "traffic": GEMM_TRAFFIC_BYTES,
-                    "traffic_unit": "bytes per launch (algorithmic: 473 MB)"}
+                    "traffic_unit": "bytes per launch, mean of the step's three products (algorithmic: 390 MB)"}
 
     out = {
         "metric": "fp8 rowwise linear fwd+bwd TFLOP/s at 7B MLP",
