@@ -14,7 +14,9 @@ Mirrors
 Differences, all deliberate:
   * single GPU: the tensor-parallel helpers (``get_splitk``, ``apply_to_partial``
     and the DTensor back-ports, lingua/float8.py:14-40,194-315) are not here;
-    the number of scale groups per row is always 1;
+    ``Fp8LinearFn`` always uses one scale group per row, while ``scale`` and
+    ``matmul`` also accept the ``[R,g]`` amaxes of the sub-row granularity those
+    helpers select under tensor parallelism;
   * forward and dgrad round to bf16 once (``bf16(acc * sa * sb + bias)``); the
     reference's dgrad rounds the unscaled product to bf16 first
     (lingua/float8.py:59-77), a work-around for a slow CUTLASS kernel;
