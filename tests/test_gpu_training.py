@@ -60,3 +60,42 @@ def test_every_variant_learns_the_batch_like_the_bf16_model():
         assert abs(got[0] - ref[0]) < 0.02 * ref[0], (kind, got[0], ref[0])
         assert got[-1] < 0.5 * got[0], (kind, got)
         assert abs(got[-1] - ref[-1]) < 0.15 * ref[-1] + 0.05, (kind, got[-1], ref[-1])
+
+
+@pytest.mark.parametrize("fused", [False, True])
+def test_activation_checkpointing_reproduces_the_plain_backward(fused):
+    """Every block under torch.utils.checkpoint (forward run again inside backward, interleaved with the
+    backward of the block after it): the quantisation memo must not hand a stale copy to the recomputed pass.
+    The kernels are deterministic, so loss and every gradient are bit-identical to the run without it."""
+    from torch.utils.checkpoint import checkpoint
+    from lingua_amd import convert_linears_to_fp8
+    from lingua_amd.callers import Llama, rope_tables
+    from lingua_amd.norm import fuse_rmsnorm
+    from lingua_amd.swiglu import fuse_feed_forward
+    with torch.device("cuda"):
+        m = Llama(**CFG).to(torch.bfloat16)
+    m.init_weights(0.04, seed=5)
+    m = convert_linears_to_fp8(m, "rowwise", r"layers\.[0-9]+\.")
+    if fused:
+        m = fuse_rmsnorm(fuse_feed_forward(m))
+    g = torch.Generator().manual_seed(6)
+    tokens = torch.randint(0, CFG["vocab"], (4, 96), generator=g).cuda()
+    labels = torch.roll(tokens, -1, dims=1)
+
+    def run(with_ac):
+        for p in m.parameters():
+            p.grad = None
+        cos, sin = rope_tables(m.head_dim, tokens.shape[1], m.rope_theta, tokens.device)
+        h = m.tok_embeddings(tokens)
+        for layer in m.layers:
+            h = checkpoint(layer, h, cos, sin, use_reentrant=False) if with_ac else layer(h, cos, sin)
+        logits = m.output(m.norm(h))
+        loss = torch.nn.functional.cross_entropy(logits.flatten(0, 1).float(), labels.flatten())
+        loss.backward()
+        return float(loss.detach()), [p.grad.clone() for p in m.parameters()]
+
+    loss_plain, grads_plain = run(False)
+    loss_ac, grads_ac = run(True)
+    assert loss_ac == loss_plain
+    for (name, _), a, b in zip(m.named_parameters(), grads_ac, grads_plain):
+        assert torch.equal(a.view(torch.int16), b.view(torch.int16)), name
