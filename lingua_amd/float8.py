@@ -152,7 +152,9 @@ class _LastCast:
     by the first backward that runs and the backward entry by the next forward."""
 
     def __init__(self):
-        self.key, self.keep, self.value, self.users = None, None, None, set()
+        # one tuple (key, tensor kept alive, value, consumers), replaced as a whole: a reader on another
+        # thread (forward and autograd threads both come here) sees either the old entry or the new one
+        self.entry = None
 
     @staticmethod
     def _key(t):
@@ -160,16 +162,17 @@ class _LastCast:
                 torch.cuda.current_stream(t.device).cuda_stream)
 
     def get(self, t, user):
-        if self.key is None or user in self.users or self.key != self._key(t):
+        entry = self.entry
+        if entry is None or user in entry[3] or entry[0] != self._key(t):
             return None
-        self.users.add(user)
-        return self.value
+        entry[3].add(user)
+        return entry[2]
 
     def put(self, t, value, user):
-        self.key, self.keep, self.value, self.users = self._key(t), t, value, {user}
+        self.entry = (self._key(t), t, value, {user})
 
     def clear(self):
-        self.key, self.keep, self.value, self.users = None, None, None, set()
+        self.entry = None
 
 
 _fwd_cast = _LastCast()   # a -> (qa, sa, a_col_amax | None)
