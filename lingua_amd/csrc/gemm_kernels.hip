@@ -74,7 +74,7 @@ L8_DEV __amdgpu_buffer_rsrc_t make_rsrc(const void *p, uint32_t bytes) {
 }
 #endif
 
-constexpr uint32_t kOOB = 0x80000000u;  // voffset that is out of range for every resource below
+[[maybe_unused]] constexpr uint32_t kOOB = 0x80000000u;  // voffset that is out of range for every resource below
 
 #ifndef L8_GEMM_DIAG
 #define L8_GEMM_DIAG 0
