@@ -21,6 +21,8 @@ import time
 ROOT = os.path.dirname(os.path.abspath(__file__))
 if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
+if os.path.join(ROOT, "tests") not in sys.path:
+    sys.path.append(os.path.join(ROOT, "tests"))   # tests/workloads.py: the stand-in Llama and the seeded inputs
 
 DIM, FFN, TOKENS = 4096, 11008, 16384
 STEP_FLOP = 18 * TOKENS * DIM * FFN          # 9 GEMMs x 2*M*N*K
@@ -180,7 +182,7 @@ def run_linear7b(args, torch, dev):
 def run_llama1b(args, torch, dev):
     """configs[4]: tokens/s of a Llama-1B-shaped forward+backward step, block linears in row-wise fp8."""
     from lingua_amd import convert_linears_to_fp8
-    from lingua_amd.callers import Llama, LLAMA_1B, llama_flops_per_token
+    from workloads import Llama, LLAMA_1B, llama_flops_per_token
     B, S = 4, 4096
     with torch.device(dev):
         model = Llama(**LLAMA_1B).to(torch.bfloat16)

@@ -49,10 +49,10 @@ int l8_device_check(int device);
  *   q        e4m3fn [R,C], row stride ldq           (may be NULL: amax only)
  *   scale    fp32 [R] = max(f32(amax),1e-12)/448    (may be NULL with q)
  *   amax     bf16 [R] row amax, NaN propagating     (may be NULL)
- *   col_amax fp32 [C] (may be NULL): max-merged (as non-negative float bit
- *            patterns) with the column amaxes of x, so that a later
- *            l8_cast_colwise_transposed() needs no pass of its own to find
- *            them.  The caller zero-fills it before the first merge.
+ *   col_amax fp32 [C] (may be NULL): receives the column amaxes of x (as
+ *            non-negative float bit patterns; overwritten, nothing to
+ *            initialise), so that a later l8_cast_colwise_transposed() needs
+ *            no pass of its own to find them.
  *   workspace  device scratch of at least l8_cast_rowwise_workspace(R, C)
  *            bytes, 16-byte aligned; needed only with col_amax (per-workgroup
  *            partial maxima, folded by a second launch on the same stream).
@@ -62,7 +62,17 @@ int l8_cast_rowwise(const void *x, int64_t R, int64_t C, int64_t ldx,
                     void *workspace, int64_t workspace_bytes, void *stream);
 int64_t l8_cast_rowwise_workspace(int64_t R, int64_t C);
 
-/* Column amax on its own (same merge semantics as col_amax above). */
+/* Row-wise scale -> cast with the row amaxes handed in, exactly as scale(t, amax_t) of
+ * lingua/float8.py:43-47 takes them: scale[r] = max(f32(amax[r]),1e-12)/448, q = e4m3(x * (1/scale)).
+ * The amax is used as given (a repeated tensor amax as at :116-118, an amax of an earlier step); where
+ * it is smaller than the row's true amax the cast behaves like the ATen one: products up to 464 round
+ * to +-448, larger ones give the NaN code.
+ *   amax bf16 [R];  q e4m3fn [R,C] (ldq);  scale fp32 [R]
+ * Requires C % 8 == 0, ldx % 8 == 0, ldq % 8 == 0, 16-byte aligned x / 8-byte aligned q. */
+int l8_cast_rowwise_given_amax(const void *x, int64_t R, int64_t C, int64_t ldx, const void *amax,
+                               void *q, int64_t ldq, float *scale, void *stream);
+
+/* Column amax on its own: col_amax fp32 [C] is overwritten, as above. */
 int l8_col_amax(const void *x, int64_t R, int64_t C, int64_t ldx, float *col_amax, void *stream);
 
 /* bf16 amax[n] -> bf16 amax_out[1] = max, NaN propagating.

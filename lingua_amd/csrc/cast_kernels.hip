@@ -15,7 +15,7 @@ namespace l8 {
 // A workgroup is 4 waves; waves stride over rows so that the optional
 // column-amax by-product is accumulated in registers over many rows, merged
 // once per workgroup in LDS and written as one row of a partial-maxima array
-// that a small second kernel folds into the caller's column amaxes.
+// that a small second kernel folds into the caller's column amaxes (overwriting them).
 // ---------------------------------------------------------------------------
 constexpr int kRowBlock = 256;
 constexpr int kRowWaves = kRowBlock / 64;
@@ -218,23 +218,39 @@ __global__ __launch_bounds__(kRowBlock, (NCHW <= 4 ? 4 : (NCHW <= 8 ? 2 : 1))) v
   }
 }
 
-// Folds the partial column maxima [n_slots, C] (bf16) into col_amax[C] (fp32 bit
-// patterns, max-merged).  Thread (x, y): column pair x, slots y*kFoldSlots .. +kFoldSlots-1.
-#ifndef L8_FOLD_SLOTS
-#define L8_FOLD_SLOTS 8
-#endif
-constexpr int kFoldSlots = L8_FOLD_SLOTS;
-__global__ __launch_bounds__(256) void colmax_fold_kernel(const uint16_t *__restrict__ partials, int n_slots, int C,
-                                                          uint32_t *__restrict__ col_amax) {
-  const int pair = blockIdx.x * 256 + threadIdx.x;
-  if (pair * 2 >= C) return;
-  const int s0 = blockIdx.y * kFoldSlots, s1 = (s0 + kFoldSlots < n_slots) ? s0 + kFoldSlots : n_slots;
+// Folds the partial column maxima [n_slots, C] (bf16, one row per workgroup of a row-wise kernel) into
+// col_amax[C] (fp32 bit patterns), which is overwritten.  A workgroup owns kFoldPairs column pairs; its
+// kFoldGroups thread groups walk interleaved slots and meet in LDS: one launch, no atomics, nothing to
+// zero beforehand.
+constexpr int kFoldPairs = 64, kFoldGroups = 16;
+__global__ __launch_bounds__(kFoldPairs *kFoldGroups) void colmax_fold_kernel(const uint16_t *__restrict__ partials,
+                                                                               int n_slots, int C,
+                                                                               uint32_t *__restrict__ col_amax) {
+  __shared__ uint32_t red[kFoldGroups][kFoldPairs];
+  const int px = threadIdx.x % kFoldPairs, sy = threadIdx.x / kFoldPairs;
+  const int pair = blockIdx.x * kFoldPairs + px;
+  const bool live = pair * 2 < C;
   uint32_t m = 0;
-  for (int sl = s0; sl < s1; ++sl)
-    m = pk_absmax_u16(m, __builtin_nontemporal_load((const uint32_t *)(partials + (int64_t)sl * C) + pair));
-  const uint32_t lo = (m & 0xffffu) << 16, hi = m & 0xffff0000u;  // bf16 -> fp32 bit patterns
-  if (lo) atomicMax(&col_amax[2 * pair], lo);
-  if (hi) atomicMax(&col_amax[2 * pair + 1], hi);
+  if (live) {
+#pragma unroll 4
+    for (int sl = sy; sl < n_slots; sl += kFoldGroups)
+      m = pk_absmax_u16(m, __builtin_nontemporal_load((const uint32_t *)(partials + (int64_t)sl * C) + pair));
+  }
+  red[sy][px] = m;
+  __syncthreads();
+  if (sy == 0 && live) {
+#pragma unroll
+    for (int g = 1; g < kFoldGroups; ++g) m = pk_absmax_u16(m, red[g][px]);
+    col_amax[2 * pair] = (m & 0xffffu) << 16;  // bf16 -> fp32 bit patterns
+    col_amax[2 * pair + 1] = m & 0xffff0000u;
+  }
+}
+
+// Zero fill for the two kernels that merge into col_amax with atomics (a kernel, not a memset, so that
+// a caller may capture the sequence in a graph).
+__global__ __launch_bounds__(256) void zero_u32_kernel(uint32_t *__restrict__ p, int64_t n) {
+  const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (i < n) p[i] = 0;
 }
 
 // Fallback for rows too long to keep in registers: two passes over the row by
@@ -353,6 +369,34 @@ __global__ __launch_bounds__(256) void cast_tensorwise_kernel(const uint16_t *__
     // the amax is handed in and must bound |x|: then every product is within
     // the finite e4m3 range and the hardware converter agrees with the ATen cast
     *(v2i *)(q + r * ldq + c) = finite ? cvt8(v, recip) : cvt8_slow(v, recip);
+  }
+}
+
+// Row-wise cast with the row amaxes handed in, as lingua/float8.py:43-47 is called: the amax is an
+// argument there, not a by-product.  It need not be the true amax of the row (a repeated tensor amax, a
+// stale amax of delayed scaling), so a product may leave the finite e4m3 range: chunks whose largest
+// product exceeds 448 take the integer conversion, which reproduces the ATen cast there (<= 464 rounds
+// to 448, above gives the NaN code).
+__global__ __launch_bounds__(256) void cast_rowwise_given_amax_kernel(const uint16_t *__restrict__ x, int64_t R, int C,
+                                                                      int64_t ldx, const uint16_t *__restrict__ amax,
+                                                                      uint8_t *__restrict__ q, int64_t ldq,
+                                                                      float *__restrict__ scale) {
+  const int cpr = C / 8;  // 16-byte chunks per row
+  const int64_t total = R * cpr;
+  for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < total; i += (int64_t)gridDim.x * 256) {
+    const int64_t r = i / cpr;
+    const int c = (int)(i - r * cpr) * 8;
+    const float s = scale_from_amax(bf16_bits_to_f32(amax[r]));  // clamp(min=EPS) also lifts a negative amax
+    const float recip = recip_exact(s);
+    if (c == 0) scale[r] = s;
+    const v4i v = __builtin_nontemporal_load((const v4i *)(x + r * ldx + c));
+    uint32_t m = 0;
+#pragma unroll
+    for (int k = 0; k < 4; ++k) m = pk_absmax_u16(m, (uint32_t)v[k]);
+    m = max(m & 0xffffu, m >> 16);
+    // !(p <= 448) also catches a NaN product (NaN element, NaN or infinite scale)
+    const float p = bf16_bits_to_f32(m) * recip;
+    *(v2i *)(q + r * ldq + c) = (p <= kE4M3Max) ? cvt8(v, recip) : cvt8_slow(v, recip);
   }
 }
 
@@ -523,8 +567,15 @@ static int64_t rowwise_blocks(int64_t R, int64_t C, bool colmax) {
 }
 
 int fold_colmax(const void *partials, int64_t slots, int64_t C, float *col_amax, hipStream_t st) {
-  hipLaunchKernelGGL(colmax_fold_kernel, dim3((unsigned)((C / 2 + 255) / 256), (unsigned)((slots + kFoldSlots - 1) / kFoldSlots)),
-                     dim3(256), 0, st, (const uint16_t *)partials, (int)slots, (int)C, (uint32_t *)col_amax);
+  hipLaunchKernelGGL(colmax_fold_kernel, dim3((unsigned)((C / 2 + kFoldPairs - 1) / kFoldPairs)),
+                     dim3(kFoldPairs * kFoldGroups), 0, st, (const uint16_t *)partials, (int)slots, (int)C,
+                     (uint32_t *)col_amax);
+  L8_HIP(hipGetLastError());
+  return L8_OK;
+}
+
+static int zero_u32(void *p, int64_t n, hipStream_t st) {
+  hipLaunchKernelGGL(zero_u32_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, st, (uint32_t *)p, n);
   L8_HIP(hipGetLastError());
   return L8_OK;
 }
@@ -601,8 +652,32 @@ extern "C" int l8_cast_rowwise(const void *x, int64_t R, int64_t C, int64_t ldx,
   if (nchw <= 8) return launch_rowwise_wg<8>(x, R, C, ldx, q, ldq, scale, amax, col_amax, ws, st);
   if (nchw <= 16) return launch_rowwise_wg<16>(x, R, C, ldx, q, ldq, scale, amax, col_amax, ws, st);
   int64_t blocks = R < (int64_t)num_cus() * 8 ? R : (int64_t)num_cus() * 8;
+  if (col_amax) {
+    const int rc = zero_u32(col_amax, C, st);
+    if (rc != L8_OK) return rc;
+  }
   hipLaunchKernelGGL(cast_rowwise_long_kernel, dim3((unsigned)blocks), dim3(kRowBlock), 0, st, (const uint16_t *)x, R,
                      (int)C, ldx, (uint8_t *)q, ldq, scale, (uint16_t *)amax, (uint32_t *)col_amax);
+  L8_HIP(hipGetLastError());
+  return L8_OK;
+}
+
+extern "C" int l8_cast_rowwise_given_amax(const void *x, int64_t R, int64_t C, int64_t ldx, const void *amax, void *q,
+                                          int64_t ldq, float *scale, void *stream) {
+  L8_REQUIRE(R >= 0 && C >= 0, "l8_cast_rowwise_given_amax: negative shape");
+  if (R == 0 || C == 0) return L8_OK;
+  L8_REQUIRE(x && amax && q && scale, "l8_cast_rowwise_given_amax: null pointer");
+  L8_REQUIRE(C % 8 == 0 && ldx % 8 == 0 && ldx >= C && aligned(x, 16),
+             "l8_cast_rowwise_given_amax: C, ldx multiples of 8 and x 16-byte aligned required");
+  L8_REQUIRE(ldq >= C && ldq % 8 == 0 && aligned(q, 8),
+             "l8_cast_rowwise_given_amax: q must be 8-byte aligned with ldq %% 8 == 0, ldq >= C");
+  L8_REQUIRE(C < (1LL << 31), "l8_cast_rowwise_given_amax: C too large");
+  const int64_t total = R * (C / 8);
+  int64_t blocks = (total + 255) / 256;
+  const int64_t cap = (int64_t)num_cus() * 16;
+  if (blocks > cap) blocks = cap;
+  hipLaunchKernelGGL(cast_rowwise_given_amax_kernel, dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream,
+                     (const uint16_t *)x, R, (int)C, ldx, (const uint16_t *)amax, (uint8_t *)q, ldq, scale);
   L8_HIP(hipGetLastError());
   return L8_OK;
 }
@@ -621,6 +696,8 @@ extern "C" int l8_col_amax(const void *x, int64_t R, int64_t C, int64_t ldx, flo
   if (rows_per < 64) rows_per = 64;
   slabs = (R + rows_per - 1) / rows_per;
   L8_REQUIRE(slabs <= 65535, "l8_col_amax: too many row slabs");
+  const int rc = zero_u32(col_amax, C, (hipStream_t)stream);
+  if (rc != L8_OK) return rc;
   hipLaunchKernelGGL(col_amax_kernel, dim3(gx, (unsigned)slabs), dim3(256), 0, (hipStream_t)stream,
                      (const uint16_t *)x, R, (int)C, ldx, (int)rows_per, (uint32_t *)col_amax);
   L8_HIP(hipGetLastError());

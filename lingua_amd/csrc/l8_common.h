@@ -33,7 +33,7 @@ constexpr int kMaxDev = 64;
 int device_slot();
 
 // Folds partial column maxima [slots, C] (bf16, one row per workgroup of a
-// row-wise kernel) into col_amax[C] (fp32 bit patterns, max-merged).  Defined in cast_kernels.hip.
+// row-wise kernel) into col_amax[C] (fp32 bit patterns, overwritten).  Defined in cast_kernels.hip.
 int fold_colmax(const void *partials, int64_t slots, int64_t C, float *col_amax, hipStream_t st);
 
 // ---- device side ----------------------------------------------------------

@@ -90,8 +90,12 @@ def scale(t: torch.Tensor, amax_t: Optional[torch.Tensor] = None):
     column groups, each with a scale of its own, which is what the reference
     computes when tensor parallelism shards the reduction dimension over ``g``
     ranks (lingua/float8.py:14-21, :86).  For the row-wise and sub-row-wise
-    cases the amax is recomputed inside the fused kernel (it is a by-product of
-    the same pass), so the values of the given tensor are not read.
+    The values of ``amax_t`` are used as given, as in the reference: a row-wise
+    amax whose rows all hold the tensor's amax (what lingua/float8.py:115-118
+    builds for dgrad) quantises tensor-wise, and an amax that is not the true
+    one (from an earlier step, say) scales by it all the same.  ``None`` asks
+    for the fused kernel that finds the row amax in the same pass; only the
+    sub-row-wise case always recomputes the group amaxes there.
     """
     if amax_t is None:
         q, s, _ = ops.cast_rowwise(t)
@@ -107,8 +111,7 @@ def scale(t: torch.Tensor, amax_t: Optional[torch.Tensor] = None):
             ops.cast_rowwise(t[:, j * cs:(j + 1) * cs], out_q=q[:, j * cs:(j + 1) * cs], out_scale=s[:, j:j + 1])
         return q, s
     if amax_t.shape[0] == t.shape[0] and t.shape[0] != 1:
-        q, s, _ = ops.cast_rowwise(t)
-        return q, s
+        return ops.cast_rowwise_given_amax(t, amax_t.to(torch.bfloat16))
     return ops.cast_tensorwise(t, amax_t.to(torch.bfloat16), transpose=False)
 
 
@@ -163,12 +166,16 @@ class _LastCast:
 
     def get(self, t, user):
         entry = self.entry
-        if entry is None or user in entry[3] or entry[0] != self._key(t):
+        # inference tensors have no version counter: nothing would show a write, so they are never shared
+        if entry is None or t.is_inference() or user in entry[3] or entry[0] != self._key(t):
             return None
         entry[3].add(user)
         return entry[2]
 
     def put(self, t, value, user):
+        if t.is_inference():
+            self.entry = None
+            return
         self.entry = (self._key(t), t, value, {user})
 
     def clear(self):
@@ -178,6 +185,17 @@ class _LastCast:
 _fwd_cast = _LastCast()   # a -> (qa, sa, a_col_amax | None)
 _bwd_cast = _LastCast()   # a -> (qat, sat)
 _fwd_tcast = _LastCast()  # a -> (qat, sat), made in forward when config.save_fp8_input
+
+
+def clear_cast_memos() -> None:
+    """Forget the shared activation casts.  The memos trust the tensor's version counter, exactly as
+    autograd's check of saved tensors does: every PyTorch in-place op and every ``out=`` write of
+    ``lingua_amd.ops`` advances it.  A write that bypasses it (``x.data.copy_``, a foreign kernel on
+    ``data_ptr()``) between two linears on the same tensor must be followed by this call (or run with
+    ``config.share_input_casts = False``)."""
+    _fwd_cast.clear()
+    _bwd_cast.clear()
+    _fwd_tcast.clear()
 
 
 def linear_forward(a, b_t, bias, need_wgrad_stats: bool, gemm_algo: int):
@@ -193,7 +211,7 @@ def linear_forward(a, b_t, bias, need_wgrad_stats: bool, gemm_algo: int):
         if not need_wgrad_stats:
             a_col_amax = None
     else:
-        a_col_amax = torch.zeros(a.shape[1], dtype=torch.float32, device=a.device) if need_wgrad_stats else None
+        a_col_amax = torch.empty(a.shape[1], dtype=torch.float32, device=a.device) if need_wgrad_stats else None
         qa, sa, _ = ops.cast_rowwise(a, col_amax=a_col_amax)
         if config.share_input_casts:
             _fwd_cast.put(a, (qa, sa, a_col_amax), b_t.data_ptr())
@@ -231,7 +249,7 @@ def linear_backward(grad_out, a, b_t, amax_b_t, a_col_amax, need_a: bool, need_b
     if need_a:
         # grad_out row-wise, weight tensor-wise from the row amaxes saved in
         # forward, quantised straight into the [K,N] layout dgrad multiplies with
-        g_col_amax = torch.zeros(grad_out.shape[1], dtype=torch.float32, device=grad_out.device) if fp8_wgrad else None
+        g_col_amax = torch.empty(grad_out.shape[1], dtype=torch.float32, device=grad_out.device) if fp8_wgrad else None
         qg, sg, _ = ops.cast_rowwise(grad_out, col_amax=g_col_amax)
         amax_b = ops.amax_reduce(amax_b_t)
         qb, sb = ops.cast_tensorwise(b_t, amax_b, transpose=True)

@@ -25,7 +25,7 @@ class Fp8RMSNormFn(torch.autograd.Function):
         if x.dtype != torch.bfloat16:
             raise RuntimeError(f"Fp8RMSNorm: bf16 activations required, got {x.dtype}")
         x2d = x.flatten(end_dim=-2)
-        col = torch.zeros(x2d.shape[1], dtype=torch.float32, device=x.device) if (training and f8.config.fp8_wgrad) else None
+        col = torch.empty(x2d.shape[1], dtype=torch.float32, device=x.device) if (training and f8.config.fp8_wgrad) else None
         y2d, q, s, rstd = ops.rmsnorm_cast_rowwise(x2d, weight, eps, want_q=True, col_amax=col, want_rstd=True)
         if f8.config.share_input_casts:
             f8._fwd_cast.put(y2d, (q, s, col), "rmsnorm")

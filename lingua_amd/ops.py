@@ -21,12 +21,19 @@ kernel_timer = None
 
 
 class _timed:
-    __slots__ = ("name", "work", "dev", "ev")
+    """Brackets one launch: makes the tensor's device current for its duration (the library launches on the
+    current device; the caller's current device is restored afterwards) and, when `kernel_timer` is a list,
+    records the two events."""
+    __slots__ = ("name", "work", "dev", "ev", "prev")
 
     def __init__(self, name, work, dev):
-        self.name, self.work, self.dev, self.ev = name, work, dev, None
+        self.name, self.work, self.dev, self.ev, self.prev = name, work, dev, None, None
 
     def __enter__(self):
+        cur = torch.cuda.current_device()
+        if self.dev.index is not None and self.dev.index != cur:
+            self.prev = cur
+            torch.cuda.set_device(self.dev)
         if kernel_timer is not None:
             self.ev = (torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True))
             self.ev[0].record(torch.cuda.current_stream(self.dev))
@@ -35,16 +42,26 @@ class _timed:
         if self.ev is not None:
             self.ev[1].record(torch.cuda.current_stream(self.dev))
             kernel_timer.append((self.name, self.ev[0], self.ev[1], self.work))
+        if self.prev is not None:
+            torch.cuda.set_device(self.prev)
         return False
 
 
 def _prep(t: torch.Tensor, what: str):
+    """Checks that `t` lives on a gfx950 GPU and returns the raw handle of the calling thread's current stream
+    on that GPU.  The process's current device is left alone."""
     if not t.is_cuda:
         raise RuntimeError(f"{what}: expected a GPU tensor, got device {t.device} (there is no CPU path)")
     _lib.require_device(t.device.index)
-    if t.device.index != torch.cuda.current_device():
-        torch.cuda.set_device(t.device)
     return torch.cuda.current_stream(t.device).cuda_stream
+
+
+def _wrote_into(t: torch.Tensor) -> None:
+    """A kernel has written into caller-supplied memory through its raw pointer: advance the tensor's version
+    counter, as an in-place PyTorch op would, so that autograd's saved-tensor check and the cast memo of
+    lingua_amd.float8 see the write."""
+    if not t.is_inference():
+        torch.autograd.graph.increment_version(t)
 
 
 def _rows_2d(t: torch.Tensor, dtype, what: str) -> torch.Tensor:
@@ -63,7 +80,7 @@ def cast_rowwise(x: torch.Tensor, col_amax: Optional[torch.Tensor] = None, want_
                  out_q: Optional[torch.Tensor] = None, out_scale: Optional[torch.Tensor] = None):
     """Row-wise amax -> scale -> e4m3fn.  Returns (q [R,C] fp8 | None, scale [R,1] fp32, amax [R,1] bf16).
 
-    ``col_amax`` (fp32 [C], zero-initialised by the caller) is max-merged with the column amaxes of x.
+    ``col_amax`` (fp32 [C]) receives the column amaxes of x (overwritten).
     ``out_q`` (fp8 [R,C], unit column stride, row stride a multiple of 8) and ``out_scale`` (fp32 [R,1], any
     strides) receive the results in place of fresh tensors: a column slice of a wider matrix is the use."""
     x = _rows_2d(x, torch.bfloat16, "cast_rowwise")
@@ -89,6 +106,8 @@ def cast_rowwise(x: torch.Tensor, col_amax: Optional[torch.Tensor] = None, want_
             amax.data_ptr(), col_amax.data_ptr() if col_amax is not None else None,
             ws.data_ptr() if ws is not None else None, ws_bytes, st)
     _lib.check(code, "l8_cast_rowwise")
+    if out_q is not None and want_q:
+        _wrote_into(out_q)
     if out_scale is not None:
         if out_scale.dtype != torch.float32 or tuple(out_scale.shape) != (R, 1):
             raise RuntimeError("cast_rowwise: out_scale must be fp32 [R,1]")
@@ -96,13 +115,33 @@ def cast_rowwise(x: torch.Tensor, col_amax: Optional[torch.Tensor] = None, want_
     return q, scale, amax
 
 
+def cast_rowwise_given_amax(x: torch.Tensor, amax: torch.Tensor):
+    """scale(x, amax) of lingua/float8.py:43-47 with a row amax [R,1] (bf16) the caller supplies and that is used as
+    given.  Returns (q [R,C] fp8, scale [R,1] fp32)."""
+    x = _rows_2d(x, torch.bfloat16, "cast_rowwise_given_amax")
+    st = _prep(x, "cast_rowwise_given_amax")
+    R, C = x.shape
+    if amax.dtype != torch.bfloat16 or amax.numel() != R or amax.device != x.device:
+        raise RuntimeError("cast_rowwise_given_amax: amax must be bf16 with one element per row, on x's device")
+    amax = amax.contiguous()
+    q = torch.empty((R, C), dtype=torch.float8_e4m3fn, device=x.device)
+    scale = torch.empty((R, 1), dtype=torch.float32, device=x.device)
+    with _timed("cast_rowwise_given_amax", R * C * 3 + 6 * R, x.device):
+        code = _lib.load().l8_cast_rowwise_given_amax(x.data_ptr(), R, C, _ld(x), amax.data_ptr(), q.data_ptr(), C,
+                                                      scale.data_ptr(), st)
+    _lib.check(code, "l8_cast_rowwise_given_amax")
+    return q, scale
+
+
 def col_amax(x: torch.Tensor) -> torch.Tensor:
     """fp32 [C] column amaxes of bf16 x [R,C]."""
     x = _rows_2d(x, torch.bfloat16, "col_amax")
     st = _prep(x, "col_amax")
     R, C = x.shape
-    out = torch.zeros(C, dtype=torch.float32, device=x.device)
-    _lib.check(_lib.load().l8_col_amax(x.data_ptr(), R, C, _ld(x), out.data_ptr(), st), "l8_col_amax")
+    out = torch.empty(C, dtype=torch.float32, device=x.device)
+    with _timed("col_amax", R * C * 2 + 4 * C, x.device):
+        code = _lib.load().l8_col_amax(x.data_ptr(), R, C, _ld(x), out.data_ptr(), st)
+    _lib.check(code, "l8_col_amax")
     return out
 
 
@@ -113,7 +152,9 @@ def amax_reduce(amax: torch.Tensor) -> torch.Tensor:
     amax = amax.contiguous()
     st = _prep(amax, "amax_reduce")
     out = torch.empty((1, 1), dtype=torch.bfloat16, device=amax.device)
-    _lib.check(_lib.load().l8_amax_reduce(amax.data_ptr(), amax.numel(), out.data_ptr(), st), "l8_amax_reduce")
+    with _timed("amax_reduce", 2 * amax.numel() + 2, amax.device):
+        code = _lib.load().l8_amax_reduce(amax.data_ptr(), amax.numel(), out.data_ptr(), st)
+    _lib.check(code, "l8_amax_reduce")
     return out
 
 
@@ -182,6 +223,7 @@ def gemm_nt(qa: torch.Tensor, qb: torch.Tensor, sa: torch.Tensor, sb: torch.Tens
         if bias.dtype != torch.bfloat16 or bias.numel() != N:
             raise RuntimeError("gemm_nt: bias must be bf16 with N elements")
         bias = bias.contiguous()
+    user_out = out is not None
     if out is None:
         out = torch.empty((M, N), dtype=torch.bfloat16, device=qa.device)
     elif out.dtype != torch.bfloat16 or out.shape != (M, N) or out.stride(1) != 1:
@@ -191,6 +233,8 @@ def gemm_nt(qa: torch.Tensor, qb: torch.Tensor, sa: torch.Tensor, sb: torch.Tens
                                       sb.data_ptr(), sb_mode, bias.data_ptr() if bias is not None else None,
                                       out.data_ptr(), _ld(out) if M > 1 else max(N, 1), algo, st)
     _lib.check(code, "l8_gemm_nt")
+    if user_out:
+        _wrote_into(out)
     return out
 
 

@@ -37,7 +37,7 @@ class Fp8SwiGLUFn(torch.autograd.Function):
         cfg = f8.config
         fp8_wgrad = cfg.fp8_wgrad
         algo = cfg.gemm_algo
-        x_col = torch.zeros(x.shape[1], dtype=torch.float32, device=x.device) \
+        x_col = torch.empty(x.shape[1], dtype=torch.float32, device=x.device) \
             if fp8_wgrad and (w1.requires_grad or w3.requires_grad) else None
         qx, sx, _ = ops.cast_rowwise(x, col_amax=x_col)
         q1, s1, amax_w1 = ops.cast_rowwise(w1)
@@ -45,7 +45,7 @@ class Fp8SwiGLUFn(torch.autograd.Function):
         h1 = ops.gemm_nt(qx, q1, sx, s1, None, algo=algo)
         h3 = ops.gemm_nt(qx, q3, sx, s3, None, algo=algo)
         del qx, q1, q3
-        h_col = torch.zeros(w2.shape[1], dtype=torch.float32, device=x.device) if fp8_wgrad and w2.requires_grad else None
+        h_col = torch.empty(w2.shape[1], dtype=torch.float32, device=x.device) if fp8_wgrad and w2.requires_grad else None
         h, qh, sh, _ = ops.swiglu_cast_rowwise(h1, h3, want_h=w2.requires_grad, col_amax=h_col)
         q2, s2, amax_w2 = ops.cast_rowwise(w2)
         y = ops.gemm_nt(qh, q2, sh, s2, None, algo=algo)
@@ -80,7 +80,7 @@ class Fp8SwiGLUFn(torch.autograd.Function):
                 gw2 = _wgrad(gy, None, h, h_col, fp8_wgrad, algo)
             return gx, gw1, gw3, gw2
 
-        gy_col = torch.zeros(D, dtype=torch.float32, device=dev) if fp8_wgrad and need_w2 else None
+        gy_col = torch.empty(D, dtype=torch.float32, device=dev) if fp8_wgrad and need_w2 else None
         qgy, sgy, _ = ops.cast_rowwise(gy, col_amax=gy_col)
         qw2t, sw2t = ops.cast_tensorwise(w2, ops.amax_reduce(amax_w2), transpose=True)
         dh = ops.gemm_nt(qgy, qw2t, sgy, sw2t, None, algo=algo)
@@ -89,8 +89,8 @@ class Fp8SwiGLUFn(torch.autograd.Function):
             gw2 = _wgrad(gy, gy_col, h, h_col, fp8_wgrad, algo)
 
         want_cols = fp8_wgrad and (need_w1 or need_w3)
-        g1_col = torch.zeros(F, dtype=torch.float32, device=dev) if want_cols else None
-        g3_col = torch.zeros(F, dtype=torch.float32, device=dev) if want_cols else None
+        g1_col = torch.empty(F, dtype=torch.float32, device=dev) if want_cols else None
+        g3_col = torch.empty(F, dtype=torch.float32, device=dev) if want_cols else None
         g1, g3, qg1, qg3, sg1, sg3 = ops.swiglu_bwd_cast_rowwise(dh, h1, h3, g1_col, g3_col)
         del dh
         if need_x:

@@ -4,9 +4,11 @@ import sys
 import pytest
 import torch
 
-ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
-if ROOT not in sys.path:
-    sys.path.insert(0, ROOT)
+HERE = os.path.dirname(os.path.abspath(__file__))
+ROOT = os.path.dirname(HERE)
+for path in (HERE, ROOT):
+    if path not in sys.path:
+        sys.path.insert(0, path)
 
 
 def pytest_configure(config):
@@ -22,12 +24,4 @@ def pytest_collection_modifyitems(config, items):
             item.add_marker(skip)
 
 
-def seeded_bf16(shape, std=1.0, seed=0):
-    """fp32 normal on the CPU generator, rounded to bf16 (identical bits for CPU oracle and GPU)."""
-    g = torch.Generator().manual_seed(seed)
-    return (torch.randn(shape, generator=g, dtype=torch.float32) * std).to(torch.bfloat16)
-
-
-def rel_l2(a: torch.Tensor, b: torch.Tensor) -> float:
-    a, b = a.detach().double().cpu(), b.detach().double().cpu()
-    return float((a - b).norm() / b.norm().clamp_min(1e-300))
+from workloads import rel_l2, seeded_bf16  # noqa: E402,F401  (tests import them from here)

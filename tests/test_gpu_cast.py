@@ -11,13 +11,18 @@ from golden_util import bits_equal, fp8_equal_mod_nan_sign, load_golden
 pytestmark = pytest.mark.gpu
 
 
+def _lib_handle():
+    from lingua_amd import _lib
+    return _lib.load()
+
+
 def dev(t):
     return t.to("cuda")
 
 
 def check_rowwise(x, with_col=False):
     from lingua_amd import ops
-    col = torch.zeros(x.shape[1], dtype=torch.float32, device="cuda") if with_col else None
+    col = torch.full((x.shape[1],), 7e29, dtype=torch.float32, device="cuda") if with_col else None   # stale contents
     q, s, a = ops.cast_rowwise(dev(x), col_amax=col)
     qo, so, ao = oracle.cast_rowwise(x)
     assert torch.equal(q.cpu().view(torch.uint8), qo), "bytes differ"
@@ -67,17 +72,26 @@ def test_rowwise_config1_inputs():
     check_rowwise(seeded_bf16((2048, 2048), 0.02, seed=1))
 
 
-def test_rowwise_strided_input_and_col_amax_merge():
+def test_rowwise_strided_input_and_col_amax_overwritten():
     from lingua_amd import ops
     big = seeded_bf16((64, 1536), seed=9)
     x = big[:, 256:256 + 1024]              # row stride 1536, offset 512 bytes
     xd = dev(big)[:, 256:256 + 1024]
-    col = torch.full((1024,), 0.5, dtype=torch.float32, device="cuda")
+    col = torch.full((1024,), 1e30, dtype=torch.float32, device="cuda")     # stale contents must not survive
     q, s, a = ops.cast_rowwise(xd, col_amax=col)
     qo, so, ao = oracle.cast_rowwise(x.contiguous())
     assert torch.equal(q.cpu().view(torch.uint8), qo) and bits_equal(s.cpu().reshape(-1), so)
-    want = torch.maximum(oracle.col_amax(x.contiguous()).float(), torch.tensor(0.5))
-    assert bits_equal(col.cpu(), want)
+    assert bits_equal(col.cpu(), oracle.col_amax(x.contiguous()).float())
+    # the stand-alone column amax and the two-pass kernel for very long rows overwrite as well
+    lib = _lib_handle()
+    col2 = torch.full((1024,), 1e30, dtype=torch.float32, device="cuda")
+    assert lib.l8_col_amax(xd.data_ptr(), 64, 1024, 1536, col2.data_ptr(), torch.cuda.current_stream().cuda_stream) == 0
+    assert bits_equal(col2.cpu(), oracle.col_amax(x.contiguous()).float())
+    wide = seeded_bf16((3, 40960), seed=10)
+    col3 = torch.full((40960,), 1e30, dtype=torch.float32, device="cuda")
+    q3, s3, _ = ops.cast_rowwise(dev(wide), col_amax=col3)
+    assert torch.equal(q3.cpu().view(torch.uint8), oracle.cast_rowwise(wide)[0])
+    assert bits_equal(col3.cpu(), oracle.col_amax(wide).float())
 
 
 def test_rowwise_nonfinite_rows():
@@ -161,18 +175,7 @@ def test_colwise_nonfinite_columns():
     assert bits_equal(s[fin], so[fin])
 
 
-def outlier_stress_input(rows=16384, cols=4096, seed=0):
-    """Student-t (df=3) activations, 0.1 % of channels x100, 1 % of rows all-zero."""
-    g = torch.Generator().manual_seed(seed)
-    z = torch.randn(rows, cols, generator=g)
-    chi = torch.randn(3, rows, cols, generator=g).pow_(2).sum(0)
-    x = z / (chi / 3.0).sqrt_()
-    del z, chi
-    ch = torch.randperm(cols, generator=g)[: max(1, cols // 1000)]
-    x[:, ch] *= 100.0
-    zr = torch.randperm(rows, generator=g)[: max(1, rows // 100)]
-    x[zr] = 0.0
-    return x.to(torch.bfloat16), ch, zr
+from workloads import outlier_stress_input  # noqa: E402
 
 
 def test_outlier_stress_full_size_rowwise_tensorwise_colwise():

@@ -109,101 +109,116 @@ def make_mlp(dim, hidden, seed):
     return layers["layers"][0], cpu_w
 
 
+def capture_linears(mlp, names=("w1", "w3", "w2")):
+    """Hooks that record, per linear, what it saw: input and output in forward, grad_out and grad_in in backward."""
+    seen, hooks = {}, []
+    for name in names:
+        lin = getattr(mlp, name)
+        hooks.append(lin.register_forward_hook(
+            lambda m_, inp, out, name=name: seen.__setitem__(name + ":io", (inp[0].detach(), out.detach()))))
+        hooks.append(lin.register_full_backward_hook(
+            lambda m_, gin, gout, name=name: seen.__setitem__(name + ":g", (gin[0].detach() if gin[0] is not None else None,
+                                                                           gout[0].detach()))))
+    return seen, hooks
+
+
 def test_config2_1b_mlp_forward_rows_vs_oracle():
-    # rows of a row-wise-scaled forward are independent: a sample of token rows pins the full-size result
+    # rows of a row-wise-scaled forward are independent: a sample of token rows pins the full-size result.  Every
+    # linear is compared with the oracle on the input the GPU handed it, so each product is held to TOL by itself.
     dim, hidden, tokens = 2048, 8192, 32768
     mlp, w = make_mlp(dim, hidden, seed=0)
     x = seeded_bf16((tokens, dim), 1.0, seed=0)
+    seen, hooks = capture_linears(mlp)
     with torch.no_grad():
         y = mlp(x.cuda().reshape(8, 4096, dim)).reshape(tokens, dim)
+    for h_ in hooks:
+        h_.remove()
     rows = torch.arange(0, tokens, tokens // 32)[:32]
+    for name in ("w1", "w3", "w2"):
+        a_in, out = (t.reshape(tokens, -1) for t in seen[name + ":io"])
+        assert rel_l2(out[rows.cuda()], oracle.linear_forward(a_in[rows.cuda()].cpu(), w[name + ".weight"])) <= TOL, name
+    assert torch.equal(seen["w1:io"][0].reshape(tokens, dim).cpu(), x)
+    # the gate between the products is PyTorch's: w2's input is silu(w1 out) * (w3 out), bit for bit
+    gate = torch.nn.functional.silu(seen["w1:io"][1]) * seen["w3:io"][1]
+    assert torch.equal(gate, seen["w2:io"][0])
+    assert torch.equal(seen["w2:io"][1].reshape(tokens, dim), y)
+    # and the chain as a whole against the oracle's own chain (three bf16 roundings deep)
     xs = x[rows]
-    x1 = oracle.linear_forward(xs, w["w1.weight"])
-    x3 = oracle.linear_forward(xs, w["w3.weight"])
-    h = torch.nn.functional.silu(x1) * x3
-    want = oracle.linear_forward(h, w["w2.weight"])
-    assert rel_l2(y[rows.cuda()], want) <= 3 * TOL   # three chained bf16 roundings; each product alone is within TOL
+    h = torch.nn.functional.silu(oracle.linear_forward(xs, w["w1.weight"])) * oracle.linear_forward(xs, w["w3.weight"])
+    assert rel_l2(y[rows.cuda()], oracle.linear_forward(h, w["w2.weight"])) <= 3 * TOL
 
 
 def test_config3_7b_mlp_forward_backward():
+    # y, dX, dW1, dW2, dW3 of the 7B MLP at full size.  Each of the three linears is compared with the oracle on the
+    # operands the GPU handed it (captured by hooks): forward and dgrad on a sample of token rows (rows are
+    # independent under row-wise scaling), wgrad on a sample of output rows x input columns (its reduction runs over
+    # every token), each within TOL.
     dim, hidden, tokens = 4096, 11008, 16384
     mlp, w = make_mlp(dim, hidden, seed=0)
     x = seeded_bf16((tokens, dim), 1.0, seed=0)
     gy = seeded_bf16((tokens, dim), 1e-2, seed=1)
     xd = x.cuda().requires_grad_(True)
-    # capture the intermediate activations / gradients the three linears see
-    seen = {}
-    hooks = []
-    for name in ("w1", "w2", "w3"):
-        lin = getattr(mlp, name)
-        hooks.append(lin.register_forward_hook(lambda m_, inp, out, name=name: seen.__setitem__(name + "_in", inp[0].detach())))
-        hooks.append(lin.register_full_backward_hook(lambda m_, gin, gout, name=name: seen.__setitem__(name + "_gout", gout[0].detach())))
+    seen, hooks = capture_linears(mlp)
     y = mlp(xd)
     y.backward(gy.cuda())
     for h_ in hooks:
         h_.remove()
     rows = torch.arange(0, tokens, tokens // 24)[:24]
-    # forward and dgrad of every linear on a row sample (rows are independent)
+    rows_d = rows.cuda()
+    dx_parts = {}
     for name in ("w1", "w3", "w2"):
         W = w[name + ".weight"]
-        a_in = seen[name + "_in"].reshape(tokens, -1)
-        g_out = seen[name + "_gout"].reshape(tokens, -1)
+        a_in, out = (t.reshape(tokens, -1) for t in seen[name + ":io"])
+        g_in, g_out = (t.reshape(tokens, -1) for t in seen[name + ":g"])
         lin = getattr(mlp, name)
-        # wgrad on a sample of output rows x input columns (the reduction runs over every token)
+        assert rel_l2(out[rows_d], oracle.linear_forward(a_in[rows_d].cpu(), W)) <= TOL, name + " forward"
+        want_dgrad = oracle.linear_dgrad(g_out[rows_d].cpu(), W)
+        assert rel_l2(g_in[rows_d], want_dgrad) <= TOL, name + " dgrad"
+        dx_parts[name] = want_dgrad
         n_idx = torch.arange(0, W.shape[0], max(1, W.shape[0] // 40))[:40]
         k_idx = torch.arange(0, W.shape[1], max(1, W.shape[1] // 40))[:40]
         qg, sg = oracle.cast_colwise_transposed(g_out[:, n_idx.cuda()].cpu())
         qa, sa = oracle.cast_colwise_transposed(a_in[:, k_idx.cuda()].cpu())
         want_dw = oracle.gemm_nt(qg, qa, sg, sa)
         got_dw = lin.weight.grad[n_idx.cuda()][:, k_idx.cuda()]
-        assert rel_l2(got_dw, want_dw) <= TOL, name
-    want_y = None
+        assert rel_l2(got_dw, want_dw) <= TOL, name + " wgrad"
+    # what the linears were handed is what the module saw: x, the gate, gy
+    assert torch.equal(seen["w1:io"][0].cpu(), x) and torch.equal(seen["w3:io"][0].cpu(), x)
+    assert torch.equal(seen["w2:g"][1].cpu(), gy) and torch.equal(seen["w2:io"][1], y.detach())
+    # dX = dgrad(w1) + dgrad(w3), added by autograd in bf16
+    want_dx = (dx_parts["w1"].float() + dx_parts["w3"].float()).to(torch.bfloat16)
+    assert xd.grad.shape == x.shape and xd.grad.dtype == torch.bfloat16
+    assert rel_l2(xd.grad[rows_d], want_dx) <= TOL
+    assert torch.isfinite(xd.grad.float()).all()
+    # y against the oracle's own chain (three bf16 roundings deep)
     xs = x[rows]
-    x1 = oracle.linear_forward(xs, w["w1.weight"])
-    x3 = oracle.linear_forward(xs, w["w3.weight"])
-    hh = torch.nn.functional.silu(x1) * x3
-    want_y = oracle.linear_forward(hh, w["w2.weight"])
-    assert rel_l2(y.detach()[rows.cuda()], want_y) <= 3 * TOL
-    # dgrad of w2 on the row sample: dh = dgrad(gy, w2)
-    dh_rows = oracle.linear_dgrad(gy[rows], w["w2.weight"])
-    # the GPU's dh is not kept by autograd; recompute it through the function for the same rows
-    from lingua_amd.float8 import Fp8LinearFn
-    hd = hh.cuda().requires_grad_(True)
-    Fp8LinearFn.apply(hd, mlp.w2.weight.detach(), None).backward(gy[rows].cuda())
-    assert rel_l2(hd.grad, dh_rows) <= TOL
-    assert xd.grad is not None and xd.grad.shape == x.shape and torch.isfinite(xd.grad.float()).all()
+    hh = torch.nn.functional.silu(oracle.linear_forward(xs, w["w1.weight"])) * oracle.linear_forward(xs, w["w3.weight"])
+    assert rel_l2(y.detach()[rows_d], oracle.linear_forward(hh, w["w2.weight"])) <= 3 * TOL
 
 
 def test_outlier_stress_rowwise_beats_tensorwise_on_the_linear():
-    # config 4: same 4096 -> 11008 linear, row-wise vs tensor-wise scaling of x and W
-    from lingua_amd import ops
-    from test_gpu_cast import outlier_stress_input
-    x, ch, zr = outlier_stress_input(rows=4096, cols=4096, seed=0)
-    w = seeded_bf16((11008, 4096), 0.02, seed=1)
-    xd, wd = x.cuda(), w.cuda()
-    qx, sx, ax = ops.cast_rowwise(xd)
-    qw, sw, aw = ops.cast_rowwise(wd)
-    y_row = ops.gemm_nt(qx, qw, sx, sw)
-    qxt, sxt = ops.cast_tensorwise(xd, ops.amax_reduce(ax))
-    qwt, swt = ops.cast_tensorwise(wd, ops.amax_reduce(aw))
-    y_ten = ops.gemm_nt(qxt, qwt, sxt, swt)
-    rows = torch.arange(0, 4096, 128)
-    want_row = oracle.gemm_nt(qx[rows.cuda()].cpu().view(torch.uint8), qw.cpu().view(torch.uint8), sx[rows.cuda()].cpu(), sw.cpu())
-    want_ten = oracle.gemm_nt(qxt[rows.cuda()].cpu().view(torch.uint8), qwt.cpu().view(torch.uint8), sxt.cpu(), swt.cpu())
-    assert rel_l2(y_row[rows.cuda()], want_row) <= TOL
-    assert rel_l2(y_ten[rows.cuda()], want_ten) <= TOL
-    exact = (xd.float() @ wd.float().t())
-    e_row = rel_l2(y_row, exact)
-    e_ten = rel_l2(y_ten, exact)
-    assert e_row < e_ten
-    assert (y_row[zr.cuda()] == 0).all()                      # all-zero token rows give exact zeros
+    # config 4 at its full 16384 tokens: both recipes against the oracle's product of the very same bytes and scales
+    # on a row sample, then the two recipes against each other
+    from workloads import outlier_stress_figures
+    fig, t = outlier_stress_figures(16384)
+    rows = torch.arange(0, 16384, 512).cuda()
+    want_row = oracle.gemm_nt(t["qx"][rows].cpu().view(torch.uint8), t["qw"].cpu().view(torch.uint8), t["sx"][rows].cpu(), t["sw"].cpu())
+    want_ten = oracle.gemm_nt(t["qxt"][rows].cpu().view(torch.uint8), t["qwt"].cpu().view(torch.uint8), t["sxt"].cpu(), t["swt"].cpu())
+    assert rel_l2(t["y_row"][rows], want_row) <= TOL
+    assert rel_l2(t["y_ten"][rows], want_ten) <= TOL
+    # and against the oracle's whole row-wise linear from the bf16 operands
+    assert rel_l2(t["y_row"][rows], oracle.linear_forward(t["x"][rows.cpu()], t["w"])) <= TOL
+    print("config 4:", fig)
+    assert fig["rel_l2_y_rowwise"] < fig["rel_l2_y_tensorwise"]
+    assert fig["snr_x_rowwise_db"] > fig["snr_x_tensorwise_db"]
+    assert (t["y_row"][t["zero_rows"].cuda()] == 0).all()        # all-zero token rows give exact zeros
 
 
 def test_config5_llama_1b_training_step():
     # full Llama-1B-shaped step (25 layers, dim 2048, 16 heads, ffn 8192, vocab 128256, 4 x 4096 tokens), all block
     # linears fp8 row-wise, output head bf16; three linears are checked against the oracle through hooks
     from lingua_amd import convert_linears_to_fp8, Fp8Linear
-    from lingua_amd.callers import Llama, LLAMA_1B
+    from workloads import Llama, LLAMA_1B
     torch.manual_seed(0)
     with torch.device("cuda"):
         model = Llama(**LLAMA_1B).to(torch.bfloat16)
@@ -302,7 +317,7 @@ def test_custom_ops_route_equals_the_autograd_function_and_compiles():
     (aot_eager: fake tensors + functionalisation + the registered autograd formula, no code generation)."""
     from lingua_amd import convert_linears_to_fp8, float8
     from lingua_amd import custom_ops
-    from lingua_amd.callers import FeedForward
+    from workloads import FeedForward
     torch.manual_seed(6)
     holder = nn.ModuleDict({"feed_forward": FeedForward(256, 512).to(device="cuda", dtype=torch.bfloat16)})
     model = convert_linears_to_fp8(holder, "rowwise", r"feed_forward\.")["feed_forward"]
@@ -364,7 +379,7 @@ def test_mlp_step_is_bitwise_reproducible():
     """No result of the path depends on scheduling: the column amaxes are max-merged (order-free), every sum runs
     in a fixed order.  Two runs of the same MLP step give identical bits, drop-in and fused."""
     from lingua_amd import convert_linears_to_fp8
-    from lingua_amd.callers import FeedForward
+    from workloads import FeedForward
     from lingua_amd.swiglu import Fp8FeedForward
     torch.manual_seed(12)
     holder = nn.ModuleDict({"feed_forward": FeedForward(512, 1536).to(device="cuda", dtype=torch.bfloat16)})
@@ -433,3 +448,113 @@ def test_fp8_copy_of_the_input_kept_for_wgrad_instead_of_the_bf16_input():
         assert rel_l2(l3.weight.grad, plain[5]) < 5e-2
     finally:
         float8.config.save_fp8_input, float8.config.fp8_wgrad = old
+
+
+def test_inference_mode_matches_no_grad():
+    """Activations made under torch.inference_mode() have no version counter (apps/main/generate.py:322 of the
+    reference generates that way): the shared-cast memo must step aside, results equal the no_grad ones."""
+    from lingua_amd import convert_linears_to_fp8
+    from lingua_amd.norm import fuse_rmsnorm
+    from workloads import TransformerBlock, rope_tables
+    torch.manual_seed(3)
+    holder = nn.ModuleDict({"layers": nn.ModuleList([TransformerBlock(256, 4, 64, 512).to(device="cuda", dtype=torch.bfloat16)])})
+    x = seeded_bf16((2, 48, 256), seed=61).cuda()
+    cos, sin = rope_tables(64, 48, 10000.0, x.device)
+    for fuse in (False, True):
+        model = convert_linears_to_fp8(holder, "rowwise", r"layers\.[0-9]+\.") if not fuse else fuse_rmsnorm(holder)
+        block = model["layers"][0]
+        with torch.no_grad():
+            want = block(x, cos, sin)
+        with torch.inference_mode():
+            xi = x * 1.0                                        # an inference tensor
+            assert xi.is_inference()
+            got = block(xi, cos, sin)
+            got2 = block(xi, cos, sin)
+        assert torch.equal(got, want) and torch.equal(got2, want)
+
+
+def test_raw_pointer_writes_are_seen_by_the_shared_casts():
+    """A kernel of this library that writes into a caller's tensor through data_ptr() advances its version counter,
+    so a linear applied afterwards does not reuse the quantised copy made before the write; writes that bypass the
+    counter (.data) are the caller's to announce with clear_cast_memos()."""
+    from lingua_amd import Fp8Linear, float8, ops
+    torch.manual_seed(9)
+    l1 = Fp8Linear(256, 256, bias=False, device="cuda", dtype=torch.bfloat16)
+    l3 = Fp8Linear(256, 256, bias=False, device="cuda", dtype=torch.bfloat16)
+    x = seeded_bf16((64, 256), seed=71).cuda()
+    other = seeded_bf16((64, 256), seed=72).cuda()
+    qa, sa, _ = ops.cast_rowwise(other)
+    qb, sb, _ = ops.cast_rowwise(l1.weight.detach())
+    with torch.no_grad():
+        l1(x)                                                   # files q(x) in the memo
+        v = x._version
+        ops.gemm_nt(qa, qb, sa, sb, out=x)                      # overwrites x in place, raw pointer
+        assert x._version > v
+        got = l3(x)
+        want = l3(x.clone())
+        assert torch.equal(got, want)
+        # the same for a cast written into a caller's buffer
+        q_user = torch.empty(64, 256, dtype=torch.float8_e4m3fn, device="cuda")
+        v = q_user._version
+        ops.cast_rowwise(other, out_q=q_user)
+        assert q_user._version > v
+        # a .data write is invisible to the version counter (to autograd's too): announce it
+        l1(x)
+        x.data.copy_(other)
+        float8.clear_cast_memos()
+        assert torch.equal(l3(x), l3(other.clone()))
+
+
+def test_selective_checkpointing_saves_the_fp8_product():
+    """lingua/distributed.py:43-50,467-473: selective activation checkpointing with the linear's forward operator in
+    the must-save list (where the reference lists aten._scaled_mm).  The recomputation in backward must not launch
+    the forward GEMMs again, and every gradient must equal the plain run bit for bit."""
+    from functools import partial
+    from torch.utils.checkpoint import CheckpointPolicy, checkpoint, create_selective_checkpoint_contexts
+    from lingua_amd import convert_linears_to_fp8, float8, ops
+    from workloads import FeedForward
+    torch.manual_seed(14)
+    holder = nn.ModuleDict({"feed_forward": FeedForward(256, 512).to(device="cuda", dtype=torch.bfloat16)})
+    mlp = convert_linears_to_fp8(holder, "rowwise", r"feed_forward\.")["feed_forward"]
+    x = seeded_bf16((4, 32, 256), seed=81).cuda()
+    gy = seeded_bf16((4, 32, 256), std=0.02, seed=82).cuda()
+    no_recompute = {torch.ops.lingua_amd.fp8_linear_fwd.default}
+
+    def policy(ctx, op, *args, **kwargs):                       # the shape of lingua/distributed.py's get_default_policy
+        return CheckpointPolicy.MUST_SAVE if op in no_recompute else CheckpointPolicy.PREFER_RECOMPUTE
+
+    def run(mode):
+        for p in mlp.parameters():
+            p.grad = None
+        xi = x.clone().requires_grad_(True)
+        rec = []
+        ops.kernel_timer = rec
+        try:
+            if mode == "plain":
+                y = mlp(xi)
+            elif mode == "sac":
+                y = checkpoint(mlp, xi, use_reentrant=False, context_fn=partial(create_selective_checkpoint_contexts, policy))
+            else:                                               # full recomputation, for the count
+                y = checkpoint(mlp, xi, use_reentrant=False)
+            n_fwd = sum(1 for r in rec if r[0] == "gemm_nt")
+            y.backward(gy)
+            n_all = sum(1 for r in rec if r[0] == "gemm_nt")
+        finally:
+            ops.kernel_timer = None
+        return [y.detach(), xi.grad] + [p.grad.clone() for p in mlp.parameters()], (n_fwd, n_all)
+
+    old = float8.config.use_custom_ops
+    float8.config.use_custom_ops = True
+    try:
+        plain, n_plain = run("plain")
+        sac, n_sac = run("sac")
+        full, n_full = run("full")
+    finally:
+        float8.config.use_custom_ops = old
+    assert n_plain == (3, 9)                                    # 3 forward products + 3 dgrads + 3 wgrads
+    assert n_sac == (3, 9), n_sac                               # nothing multiplied twice: the products were saved
+    assert n_full == (3, 12), n_full                            # plain checkpointing runs the three forwards again
+    for a, b in zip(sac, plain):
+        assert torch.equal(a.view(torch.int16), b.view(torch.int16))
+    for a, b in zip(full, plain):
+        assert torch.equal(a.view(torch.int16), b.view(torch.int16))

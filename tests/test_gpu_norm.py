@@ -100,7 +100,7 @@ class _Block(torch.nn.Module):
 
     def __init__(self, dim):
         super().__init__()
-        from lingua_amd.callers import RMSNorm
+        from workloads import RMSNorm
         self.attention_norm = RMSNorm(dim, EPS)
         self.wq = torch.nn.Linear(dim, dim, bias=False)
         self.wk = torch.nn.Linear(dim, dim // 2, bias=False)
@@ -163,7 +163,7 @@ def test_small_llama_with_fused_gate_and_norms_matches_the_drop_in_model():
     models are not compared with each other directly: each gradient of the fused model must be as close to the
     bf16 model's as the drop-in model's is (within a quarter more), and the losses must agree."""
     from lingua_amd import convert_linears_to_fp8
-    from lingua_amd.callers import Llama
+    from workloads import Llama
     from lingua_amd.norm import Fp8RMSNorm, fuse_rmsnorm
     from lingua_amd.swiglu import Fp8FeedForward, fuse_feed_forward
     cfg = dict(n_layers=3, dim=512, n_heads=4, ffn_dim=1536, vocab=1000)

@@ -65,3 +65,59 @@ def test_rejected_tilings():
         f8.scale(x, torch.ones(1, 2, device="cuda"))
     with pytest.raises(RuntimeError, match="column groups"):
         f8.matmul(x, torch.ones(8, 2, device="cuda"), x, torch.ones(8, 3, device="cuda"), None)
+
+
+def test_scale_uses_the_row_amax_it_is_given():
+    """scale(t, amax [R,1]) multiplies by 448 / amax of the ARGUMENT (lingua/float8.py:43-47): the true amax gives the
+    fused kernel's bytes, a repeated tensor amax (what lingua/float8.py:115-118 builds) gives the tensor-wise bytes,
+    and an amax below the true one saturates / overflows as the ATen cast does."""
+    from golden_util import fp8_equal_mod_nan_sign
+    from lingua_amd import float8 as f8, ops
+    x = seeded_bf16((300, 1024), std=2.0, seed=77)
+    x[5] = 0.0
+    x[7, 100] = 3000.0
+    xd = x.cuda()
+    true_amax = rt.row_amax(x)
+    # (1) the true amax: same bytes and scales as the fused kernel and as the oracle
+    q, s = f8.scale(xd, true_amax.cuda())
+    qf, sf, _ = ops.cast_rowwise(xd)
+    qo, so, _ = oracle.cast_rowwise(x)
+    assert torch.equal(q.view(torch.uint8), qf.view(torch.uint8)) and bits_equal(s, sf)
+    assert torch.equal(q.cpu().view(torch.uint8), qo) and bits_equal(s.cpu().reshape(-1), so)
+    # (2) every row holds the tensor amax: the tensor-wise quantisation
+    rep = true_amax.amax().reshape(1, 1).repeat(300, 1)
+    q2, s2 = f8.scale(xd, rep.cuda())
+    qt, st_ = oracle.cast_tensorwise(x)
+    assert torch.equal(q2.cpu().view(torch.uint8), qt)
+    assert bits_equal(s2.cpu().reshape(-1), st_.repeat(300))
+    # (3) an amax that is too small (a quarter of the true one), a negative one and a zero one: the PyTorch op chain
+    wrong = (true_amax.float() / 4).to(torch.bfloat16)
+    wrong[9] = -1.0
+    wrong[11] = 0.0
+    q3, s3 = f8.scale(xd, wrong.cuda())
+    want_q, want_s = rt.scale(x, wrong)
+    assert fp8_equal_mod_nan_sign(q3, want_q) and bits_equal(s3.cpu(), want_s)
+    codes = q3.cpu().view(torch.uint8) & 0x7F
+    assert (codes == 0x7F).any() and (codes == 0x7E).any()       # both the NaN code and the clipped 448 occur
+    # (4) non-finite amaxes
+    bad = true_amax.clone()
+    bad[1], bad[2] = float("inf"), float("nan")
+    q4, s4 = f8.scale(xd, bad.cuda())
+    want_q, want_s = rt.scale(x, bad)
+    assert fp8_equal_mod_nan_sign(q4, want_q) and bits_equal(s4.cpu(), want_s)
+
+
+def test_matmul_called_as_the_reference_dgrad_calls_it():
+    """lingua/float8.py:110-119: grad_out with its row amax, the transposed weight with its tensor amax repeated
+    over the rows.  The public matmul() must honour that amax and give the oracle's dgrad."""
+    from lingua_amd import float8 as f8
+    M, K, N = 200, 256, 384
+    g = seeded_bf16((M, N), std=1e-2, seed=5)
+    w = seeded_bf16((N, K), std=0.02, seed=6)
+    w[3, 10] = 1.0                                             # one large weight: row-wise and tensor-wise differ
+    b = w.t().contiguous()                                     # [K,N], what lingua/float8.py:111 makes
+    amax_b = rt.tensor_amax_from_rows(rt.row_amax(w), K)       # [K,1], every row the tensor amax
+    got = f8.matmul(g.cuda(), rt.row_amax(g).cuda(), b.cuda(), amax_b.cuda(), None, use_fast_accum=False)
+    assert rel_l2(got, oracle.linear_dgrad(g, w)) <= 1e-3
+    rowwise_b = f8.matmul(g.cuda(), rt.row_amax(g).cuda(), b.cuda(), rt.row_amax(b).cuda(), None)
+    assert not torch.equal(got, rowwise_b)

@@ -5,7 +5,9 @@ the same layers (wq/wk/wv/wo/w1/w2/w3 in every block, not ``output`` /
 
 They exist so that tests and benchmarks can drive ``convert_linears_to_fp8``
 the way lingua's ``parallelize_model`` does (lingua/distributed.py:403-406);
-everything that is not a linear runs on plain PyTorch ops.
+everything that is not a linear runs on plain PyTorch ops.  Also here: the
+seeded synthetic inputs that tests and benchmark share.  Not part of the
+product package.
 
   * ``FeedForward``      SwiGLU MLP, lingua/transformer.py:430-471
   * ``Attention``        lingua/transformer.py:306-410 (causal sdpa path only)
@@ -128,3 +130,61 @@ def llama_flops_per_token(n_layers: int, dim: int, ffn_dim: int, vocab: int, seq
 
 
 LLAMA_1B = dict(n_layers=25, dim=2048, n_heads=16, ffn_dim=8192, vocab=128256)
+
+
+# ----------------------------------------------------------------------------
+# seeded synthetic inputs shared by the tests and the benchmark
+# ----------------------------------------------------------------------------
+
+def seeded_bf16(shape, std=1.0, seed=0):
+    """fp32 normal on the CPU generator, rounded to bf16 (identical bits for CPU oracle and GPU)."""
+    g = torch.Generator().manual_seed(seed)
+    return (torch.randn(shape, generator=g, dtype=torch.float32) * std).to(torch.bfloat16)
+
+
+def rel_l2(a: torch.Tensor, b: torch.Tensor) -> float:
+    a, b = a.detach().double().cpu(), b.detach().double().cpu()
+    return float((a - b).norm() / b.norm().clamp_min(1e-300))
+
+
+def outlier_stress_input(rows=16384, cols=4096, seed=0):
+    """Student-t (df=3) activations, 0.1 % of channels x100, 1 % of rows all-zero."""
+    g = torch.Generator().manual_seed(seed)
+    z = torch.randn(rows, cols, generator=g)
+    chi = torch.randn(3, rows, cols, generator=g).pow_(2).sum(0)
+    x = z / (chi / 3.0).sqrt_()
+    del z, chi
+    ch = torch.randperm(cols, generator=g)[: max(1, cols // 1000)]
+    x[:, ch] *= 100.0
+    zr = torch.randperm(rows, generator=g)[: max(1, rows // 100)]
+    x[zr] = 0.0
+    return x.to(torch.bfloat16), ch, zr
+
+
+def outlier_stress_figures(tokens: int = 16384):
+    """The 4096 -> 11008 linear on the outlier-stress activations, row-wise against tensor-wise scaling of both
+    operands.  Returns the reported figures -- quantisation SNR of x (dB) and rel-L2 of the output against the fp32
+    product of the unquantised operands, for either recipe -- and the GPU tensors they were computed from."""
+    from lingua_amd import ops
+    x, ch, zr = outlier_stress_input(rows=tokens, cols=4096, seed=0)
+    w = seeded_bf16((11008, 4096), 0.02, seed=1)
+    xd, wd = x.cuda(), w.cuda()
+    qx, sx, ax = ops.cast_rowwise(xd)
+    qw, sw, aw = ops.cast_rowwise(wd)
+    y_row = ops.gemm_nt(qx, qw, sx, sw)
+    qxt, sxt = ops.cast_tensorwise(xd, ops.amax_reduce(ax))
+    qwt, swt = ops.cast_tensorwise(wd, ops.amax_reduce(aw))
+    y_ten = ops.gemm_nt(qxt, qwt, sxt, swt)
+    exact = xd.float() @ wd.float().t()
+
+    def snr_db(q, s):
+        err = (q.float() * s - xd.float()).double().pow(2).sum()
+        return 10.0 * math.log10(float(xd.double().pow(2).sum() / err))
+
+    def err(y):
+        return float((y.double() - exact.double()).norm() / exact.double().norm())
+
+    figures = {"tokens": tokens, "snr_x_rowwise_db": round(snr_db(qx, sx), 2), "snr_x_tensorwise_db": round(snr_db(qxt, sxt), 2),
+               "rel_l2_y_rowwise": float(f"{err(y_row):.4e}"), "rel_l2_y_tensorwise": float(f"{err(y_ten):.4e}")}
+    return figures, dict(x=x, w=w, zero_rows=zr, qx=qx, sx=sx, qw=qw, sw=sw, qxt=qxt, sxt=sxt, qwt=qwt, swt=swt,
+                         y_row=y_row, y_ten=y_ten)
