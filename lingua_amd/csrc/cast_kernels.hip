@@ -623,24 +623,18 @@ extern "C" int64_t l8_cast_rowwise_workspace(int64_t R, int64_t C) {
   return rowwise_blocks(R, C, true) * C * (int64_t)sizeof(uint16_t);
 }
 
-extern "C" int l8_cast_rowwise(const void *x, int64_t R, int64_t C, int64_t ldx, void *q, int64_t ldq, float *scale,
-                               void *amax, float *col_amax, void *workspace, int64_t workspace_bytes, void *stream) {
-  L8_REQUIRE(R >= 0 && C >= 0, "l8_cast_rowwise: negative shape R=%lld C=%lld", (long long)R, (long long)C);
-  if (R == 0 || C == 0) return L8_OK;
-  L8_REQUIRE(x != nullptr, "l8_cast_rowwise: x is null");
-  L8_REQUIRE((q == nullptr) || (scale != nullptr), "l8_cast_rowwise: q given without scale");
-  L8_REQUIRE(C % 8 == 0 && ldx % 8 == 0 && ldx >= C, "l8_cast_rowwise: C=%lld and ldx=%lld must be multiples of 8, ldx >= C",
+// Argument checks and dispatch shared by l8_cast_rowwise and l8_cast_rowwise_noalloc; `what` names the
+// entry point in error messages.  `workspace` holds at least l8_cast_rowwise_workspace(R, C) bytes when
+// col_amax is given (checked by the callers).
+static int cast_rowwise_impl(const char *what, const void *x, int64_t R, int64_t C, int64_t ldx, void *q, int64_t ldq,
+                             float *scale, void *amax, float *col_amax, void *workspace, hipStream_t st) {
+  L8_REQUIRE(x != nullptr, "%s: x is null", what);
+  L8_REQUIRE((q == nullptr) || (scale != nullptr), "%s: q given without scale", what);
+  L8_REQUIRE(C % 8 == 0 && ldx % 8 == 0 && ldx >= C, "%s: C=%lld and ldx=%lld must be multiples of 8, ldx >= C", what,
              (long long)C, (long long)ldx);
-  L8_REQUIRE(aligned(x, 16), "l8_cast_rowwise: x must be 16-byte aligned");
-  if (q) L8_REQUIRE(ldq % 8 == 0 && ldq >= C && aligned(q, 8), "l8_cast_rowwise: q must be 8-byte aligned with ldq %% 8 == 0, ldq >= C");
-  L8_REQUIRE(C < (1LL << 31), "l8_cast_rowwise: C too large");
-  if (col_amax) {
-    const int64_t need = l8_cast_rowwise_workspace(R, C);
-    L8_REQUIRE(need == 0 || (workspace != nullptr && workspace_bytes >= need && aligned(workspace, 16)),
-               "l8_cast_rowwise: col_amax needs a 16-byte aligned workspace of %lld bytes (l8_cast_rowwise_workspace)",
-               (long long)need);
-  }
-  hipStream_t st = (hipStream_t)stream;
+  L8_REQUIRE(aligned(x, 16), "%s: x must be 16-byte aligned", what);
+  if (q) L8_REQUIRE(ldq % 8 == 0 && ldq >= C && aligned(q, 8), "%s: q must be 8-byte aligned with ldq %% 8 == 0, ldq >= C", what);
+  L8_REQUIRE(C < (1LL << 31), "%s: C too large", what);
   void *ws = workspace;
   const int64_t nch = (C + 511) / 512;
   if (nch <= 4) return launch_rowwise<4>(x, R, C, ldx, q, ldq, scale, amax, col_amax, ws, st);
@@ -660,6 +654,19 @@ extern "C" int l8_cast_rowwise(const void *x, int64_t R, int64_t C, int64_t ldx,
                      (int)C, ldx, (uint8_t *)q, ldq, scale, (uint16_t *)amax, (uint32_t *)col_amax);
   L8_HIP(hipGetLastError());
   return L8_OK;
+}
+
+extern "C" int l8_cast_rowwise(const void *x, int64_t R, int64_t C, int64_t ldx, void *q, int64_t ldq, float *scale,
+                               void *amax, float *col_amax, void *workspace, int64_t workspace_bytes, void *stream) {
+  L8_REQUIRE(R >= 0 && C >= 0, "l8_cast_rowwise: negative shape R=%lld C=%lld", (long long)R, (long long)C);
+  if (R == 0 || C == 0) return L8_OK;
+  if (col_amax) {
+    const int64_t need = l8_cast_rowwise_workspace(R, C);
+    L8_REQUIRE(need == 0 || (workspace != nullptr && workspace_bytes >= need && aligned(workspace, 16)),
+               "l8_cast_rowwise: col_amax needs a 16-byte aligned workspace of %lld bytes (l8_cast_rowwise_workspace)",
+               (long long)need);
+  }
+  return cast_rowwise_impl("l8_cast_rowwise", x, R, C, ldx, q, ldq, scale, amax, col_amax, workspace, (hipStream_t)stream);
 }
 
 extern "C" int l8_cast_rowwise_given_amax(const void *x, int64_t R, int64_t C, int64_t ldx, const void *amax, void *q,
