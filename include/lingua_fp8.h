@@ -62,6 +62,23 @@ int l8_cast_rowwise(const void *x, int64_t R, int64_t C, int64_t ldx,
                     void *workspace, int64_t workspace_bytes, void *stream);
 int64_t l8_cast_rowwise_workspace(int64_t R, int64_t C);
 
+/* l8_cast_rowwise for callers that cannot allocate device memory (code under HIP graph capture, tight
+ * serving loops, harnesses that forbid hipMalloc).  No counterpart in the reference, whose ATen ops
+ * allocate freely.  Same arguments and results as l8_cast_rowwise without the workspace: the partial
+ * column maxima go to a static device array of L8_NOALLOC_SCRATCH_BYTES that every GPU the library runs
+ * on holds until the process ends.  Calls no allocator.
+ *   - shapes whose l8_cast_rowwise_workspace(R, C) exceeds L8_NOALLOC_SCRATCH_BYTES are rejected
+ *     (L8_EINVAL) when col_amax is given: with 256 compute units that is C > 16384 together with
+ *     R >= 512; without col_amax no scratch is used and any shape goes;
+ *   - all calls on one GPU share that GPU's array: two calls with col_amax that overlap in time on the
+ *     same GPU (different streams or threads) race.  Nothing in it needs clearing between calls: every
+ *     call writes the part it reads.
+ *   - the array's address is looked up once per device, by l8_device_check(device) or else by the first
+ *     call on that device; call l8_device_check before capturing. */
+#define L8_NOALLOC_SCRATCH_BYTES (16 * 1024 * 1024)
+int l8_cast_rowwise_noalloc(const void *x, int64_t R, int64_t C, int64_t ldx,
+                            void *q, int64_t ldq, float *scale, void *amax, float *col_amax, void *stream);
+
 /* Row-wise scale -> cast with the row amaxes handed in, exactly as scale(t, amax_t) of
  * lingua/float8.py:43-47 takes them: scale[r] = max(f32(amax[r]),1e-12)/448, q = e4m3(x * (1/scale)).
  * The amax is used as given (a repeated tensor amax as at :116-118, an amax of an earlier step); where

@@ -22,6 +22,7 @@ SIGNATURES = {
     "l8_device_check": [_int],
     "l8_cast_rowwise": [_p, _i64, _i64, _i64, _p, _i64, _p, _p, _p, _p, _i64, _p],
     "l8_cast_rowwise_workspace": [_i64, _i64],
+    "l8_cast_rowwise_noalloc": [_p, _i64, _i64, _i64, _p, _i64, _p, _p, _p, _p],
     "l8_cast_rowwise_given_amax": [_p, _i64, _i64, _i64, _p, _p, _i64, _p, _p],
     "l8_col_amax": [_p, _i64, _i64, _i64, _p, _p],
     "l8_amax_reduce": [_p, _i64, _p, _p],

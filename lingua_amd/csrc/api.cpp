@@ -48,5 +48,14 @@ extern "C" int l8_device_check(int device) {
   if (e != hipSuccess) return l8::fail(L8_EHIP, "hipGetDeviceProperties(%d): %s", device, hipGetErrorString(e));
   if (strncmp(prop.gcnArchName, "gfx950", 6) != 0)
     return l8::fail(L8_EARCH, "device %d is %s; this library contains gfx950 code only", device, prop.gcnArchName);
-  return L8_OK;
+  // per-device set-up, with that device current for its duration
+  int prev = -1;
+  if (hipGetDevice(&prev) != hipSuccess) prev = -1;
+  if (prev != device) {
+    e = hipSetDevice(device);
+    if (e != hipSuccess) return l8::fail(L8_EHIP, "hipSetDevice(%d): %s", device, hipGetErrorString(e));
+  }
+  const int rc = l8::noalloc_setup_current_device();
+  if (prev != device && prev >= 0) (void)hipSetDevice(prev);
+  return rc;
 }

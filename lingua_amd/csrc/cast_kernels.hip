@@ -4,6 +4,9 @@
 // amax reductions at :86-87 / :112-114, the tensor amax at :115-118 and the
 // weight transpose copy at :111.  Compulsory traffic per element is 2 bytes
 // read + 1 byte written; every kernel here reads each input byte from HBM once.
+#include <atomic>
+#include <mutex>
+
 #include "l8_common.h"
 
 namespace l8 {
@@ -667,6 +670,58 @@ extern "C" int l8_cast_rowwise(const void *x, int64_t R, int64_t C, int64_t ldx,
                (long long)need);
   }
   return cast_rowwise_impl("l8_cast_rowwise", x, R, C, ldx, q, ldq, scale, amax, col_amax, workspace, (hipStream_t)stream);
+}
+
+// ---------------------------------------------------------------------------
+// l8_cast_rowwise for callers that cannot allocate: the partial column maxima go to a static device
+// array instead of a caller-supplied workspace.  Each GPU holds its own copy of the array at its own
+// address; the address is looked up once per device (with that device current) and kept.
+// ---------------------------------------------------------------------------
+static __device__ __align__(256) unsigned char scratch[L8_NOALLOC_SCRATCH_BYTES];
+static std::atomic<void *> g_scratch_ptr[l8::kMaxDev];  // device address of `scratch`, per device
+static std::mutex g_scratch_mutex;
+
+// Device address of `scratch` on the current device (looked up on first use).
+static int scratch_of_current_device(void **out) {
+  int dev = -1;
+  L8_HIP(hipGetDevice(&dev));
+  L8_REQUIRE(dev >= 0 && dev < kMaxDev, "device ordinal %d beyond the %d this library keeps state for", dev, kMaxDev);
+  void *ptr = g_scratch_ptr[dev].load(std::memory_order_acquire);
+  if (!ptr) {
+    std::lock_guard<std::mutex> lock(g_scratch_mutex);
+    ptr = g_scratch_ptr[dev].load(std::memory_order_relaxed);
+    if (!ptr) {
+      L8_HIP(hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)));
+      L8_REQUIRE(ptr != nullptr, "hipGetSymbolAddress returned a null address for the scratch array");
+      g_scratch_ptr[dev].store(ptr, std::memory_order_release);
+    }
+  }
+  *out = ptr;
+  return L8_OK;
+}
+
+// Called by l8_device_check with `device` current, so that the look-up (which may load the code object)
+// happens at set-up and not inside a caller's capture or serving loop.
+int l8::noalloc_setup_current_device() {
+  void *ptr = nullptr;
+  return scratch_of_current_device(&ptr);
+}
+
+extern "C" int l8_cast_rowwise_noalloc(const void *x, int64_t R, int64_t C, int64_t ldx, void *q, int64_t ldq,
+                                       float *scale, void *amax, float *col_amax, void *stream) {
+  L8_REQUIRE(R >= 0 && C >= 0, "l8_cast_rowwise_noalloc: negative shape R=%lld C=%lld", (long long)R, (long long)C);
+  if (R == 0 || C == 0) return L8_OK;
+  void *ws = nullptr;
+  if (col_amax) {
+    const int64_t need = l8_cast_rowwise_workspace(R, C);
+    L8_REQUIRE(need <= (int64_t)L8_NOALLOC_SCRATCH_BYTES,
+               "l8_cast_rowwise_noalloc: [%lld,%lld] with column amaxes needs %lld bytes of scratch, the static array "
+               "holds %lld (use l8_cast_rowwise with a workspace)",
+               (long long)R, (long long)C, (long long)need, (long long)L8_NOALLOC_SCRATCH_BYTES);
+    const int rc = scratch_of_current_device(&ws);
+    if (rc != L8_OK) return rc;
+  }
+  return cast_rowwise_impl("l8_cast_rowwise_noalloc", x, R, C, ldx, q, ldq, scale, amax, col_amax, ws, (hipStream_t)stream);
 }
 
 extern "C" int l8_cast_rowwise_given_amax(const void *x, int64_t R, int64_t C, int64_t ldx, const void *amax, void *q,

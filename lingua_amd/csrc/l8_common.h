@@ -36,6 +36,10 @@ int device_slot();
 // row-wise kernel) into col_amax[C] (fp32 bit patterns, overwritten).  Defined in cast_kernels.hip.
 int fold_colmax(const void *partials, int64_t slots, int64_t C, float *col_amax, hipStream_t st);
 
+// Looks up, for the current device, the address of the static scratch array of l8_cast_rowwise_noalloc.
+// Defined in cast_kernels.hip; l8_device_check calls it so that the look-up happens at set-up.
+int noalloc_setup_current_device();
+
 // ---- device side ----------------------------------------------------------
 #define L8_DEV __device__ __forceinline__
 
