@@ -62,6 +62,7 @@ struct GemmArgs {
   const uint16_t *bias;
   uint16_t *C;
   int tiles_m, tiles_n;
+  uint64_t *dbg;  // L8_GEMM_PROF builds only
 };
 
 typedef __attribute__((address_space(3))) void *lds_ptr_t;
@@ -81,6 +82,12 @@ L8_DEV __amdgpu_buffer_rsrc_t make_rsrc(const void *p, uint32_t bytes) {
 #endif
 #ifndef L8_STRADDLE
 #define L8_STRADDLE 2
+#endif
+// L8_GEMM_PROF (compile-time, never set in the shipped build): the persistent kernel takes the `bias` pointer for
+// a buffer of 16 x uint64 per workgroup and records wall-clock ticks (100 MHz) at its start, after the prologue
+// and at its end, and shader-clock cycles spent in the K loops and in the C-tile stores.
+#ifndef L8_GEMM_PROF
+#define L8_GEMM_PROF 0
 #endif
 
 // s_waitcnt for vmcnt <= n and lgkmcnt == 0 (expcnt untouched)
@@ -476,6 +483,380 @@ __global__ __launch_bounds__(WM *WN * 64) void gemm_nt_kernel(const GemmArgs p) 
 }
 
 // ---------------------------------------------------------------------------
+// Persistent variant for large problems: one workgroup per compute unit walks a
+// list of 256x256 tiles, and the panel stream (global -> LDS ring) runs on
+// from the last K tile of one output tile into the first K tiles of the next,
+// so that only the very first tile of a workgroup pays a prologue.
+//
+// The C tile leaves straight from the accumulators, with no staging in LDS
+// (the ring stays in use by the panel stream) and no barrier:
+//   * the matrix cores compute D[i = m][j = n'] (A rows on the first port);
+//   * LDS row tn*32 + j of a wave's 128-row span of the B panel holds the
+//     global B row 4*j + tn of that span (the permutation is applied on the
+//     global-address side of the direct-to-LDS loads, which is free), so that
+//     lane j owns, at the same accumulator index of its four tn tiles, the
+//     four CONSECUTIVE output columns 4*j .. 4*j+3;
+//   * one 8-byte store per lane then covers 256 contiguous bytes of a C row
+//     per half-wave (two rows per wave instruction, whole 128-byte lines).
+// Work split: the tiles are dealt to the 8 XCDs in contiguous ranges of the
+// grouped order (as in the kernel above); inside an XCD, workgroup `loc`
+// takes tiles loc, loc + W, loc + 2W, ... of the range (W workgroups per XCD),
+// so the workgroups resident on an XCD always work on W consecutive tiles of
+// the grouped order and share their panels in that XCD's L2.
+// ---------------------------------------------------------------------------
+template <int GROUP_M, bool HAS_BIAS>
+__global__ __launch_bounds__(256) void gemm_nt_stream_kernel(const GemmArgs p) {
+#if defined(__HIP_DEVICE_COMPILE__)
+  constexpr int BM = 256, BN = 256, BK = 128, NW = 4, TM = 4, TN = 4, R = 5;
+  constexpr int UNIT = BM * BK;    // one ring slot: the A or the B panel of one K tile
+  constexpr int NL = BM / 8 / NW;  // 1 KiB wave loads (8 rows x 128 B) per panel per wave
+  constexpr int PEND = NL;         // in flight at the barrier of a trip: the unit requested in its first half
+  constexpr int PEND0 = 2 * NL;    // prologue: K tile 1 may be in flight when K tile 0 is published
+  constexpr int N_STORES = TM * 4 * 2;  // store instructions per wave and C tile
+  static_assert(N_STORES + PEND <= 63, "vmcnt is a 6-bit counter");
+  extern __shared__ __attribute__((aligned(1024))) uint8_t smem[];
+
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int wm = wave >> 1, wn = wave & 1;
+
+  // ---- this workgroup's tiles ----
+  const int nb = p.tiles_m * p.tiles_n;
+  const int xcd = blockIdx.x & 7, loc = blockIdx.x >> 3, W = gridDim.x >> 3;
+  const int q = nb >> 3, rem = nb & 7;
+  const int first = (xcd < rem) ? xcd * (q + 1) : rem * (q + 1) + (xcd - rem) * q;
+  const int cnt = q + (xcd < rem ? 1 : 0);
+  const int n_seg = loc < cnt ? (cnt - loc + W - 1) / W : 0;
+  if (n_seg == 0) return;
+  [[maybe_unused]] uint64_t prof[16] = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+  const int KT = (p.K + BK - 1) / BK;
+  auto tile_of = [&](int seg, int &m0, int &n0) {
+    const int lin = first + loc + seg * W;
+    const int per_group = GROUP_M * p.tiles_n;
+    const int grp = lin / per_group;
+    const int first_m = grp * GROUP_M;
+    const int gsz = (p.tiles_m - first_m < GROUP_M) ? p.tiles_m - first_m : GROUP_M;
+    const int in_grp = lin - grp * per_group;
+    m0 = (first_m + in_grp % gsz) * BM;
+    n0 = (in_grp / gsz) * BN;
+  };
+
+  // ---- global -> LDS load plan ----
+  // lane l of a wave load fills LDS row l/8, position l%8 of an 8-row group; position p of LDS row r holds
+  // chunk p ^ f(r), f(r) = (r & 7) ^ ((r >> 3) & 1).  Wave load i of a panel fills the LDS rows of group
+  // g = wave * NL + i.  For the A panel LDS row = tile row.  For the B panel LDS row r = span*128 + tn*32 + j
+  // holds tile row span*128 + 4*j + tn: within a group (8 consecutive j) the rows are 4 apart, and the
+  // group's first row is span*128 + 4*(8*(g%4)) + (g%16)/4.
+  const int lrow = lane >> 3, lpos = lane & 7;
+  const uint32_t a_voff[2] = {(uint32_t)(lrow * (int)p.lda + (lpos ^ lrow) * 16), (uint32_t)(lrow * (int)p.lda + (lpos ^ lrow ^ 1) * 16)};
+  const uint32_t b_voff[2] = {(uint32_t)(lrow * 4 * (int)p.ldb + (lpos ^ lrow) * 16), (uint32_t)(lrow * 4 * (int)p.ldb + (lpos ^ lrow ^ 1) * 16)};
+  const int chunk_even = (lpos ^ lrow) * 16, chunk_odd = (lpos ^ lrow ^ 1) * 16;
+  const uint32_t lds0 = (uint32_t)(uintptr_t)(lds_ptr_t)smem;
+  auto wrap = [](int slot) { return slot >= R ? slot - R : slot; };
+
+  // loader cursor: the K tile whose panels are requested next (two K tiles ahead of the one being multiplied)
+  int ld_seg = 0, ld_kt = 0;
+  __amdgpu_buffer_rsrc_t ld_rsA, ld_rsB;
+  auto ld_open = [&](int seg) {
+    if (seg < n_seg) {
+      int m0, n0;
+      tile_of(seg, m0, n0);
+      const int64_t a_left = (int64_t)(p.M - m0 - 1) * p.lda + p.K;
+      const int64_t b_left = (int64_t)(p.N - n0 - 1) * p.ldb + p.K;
+      ld_rsA = make_rsrc(p.A + (int64_t)m0 * p.lda, a_left < 0x7fffffff ? (uint32_t)a_left : 0x7fffffffu);
+      ld_rsB = make_rsrc(p.B + (int64_t)n0 * p.ldb, b_left < 0x7fffffff ? (uint32_t)b_left : 0x7fffffffu);
+    } else {  // past the last tile: every load is out of range and fills its LDS bytes with zeros
+      ld_rsA = make_rsrc(p.A, 0);
+      ld_rsB = make_rsrc(p.B, 0);
+    }
+  };
+  auto ld_advance = [&]() {
+    if (++ld_kt == KT) {
+      ld_kt = 0;
+      ld_open(++ld_seg);
+    }
+  };
+  // i-th wave load (of NL) of the A or B panel of the loader's K tile into ring slot `slot`
+  auto load_one = [&](bool is_b, int slot, int i) {
+    const int k0 = ld_kt * BK;
+    const uint32_t m_even = (k0 + chunk_even < p.K) ? 0u : kOOB, m_odd = (k0 + chunk_odd < p.K) ? 0u : kOOB;
+    const uint32_t dst = lds0 + slot * UNIT + (wave * NL + i) * 1024;
+    if (!is_b) {
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(ld_rsA, reinterpret_cast<lds_ptr_t>(dst), 16, a_voff[i & 1] | ((i & 1) ? m_odd : m_even),
+                                               k0 + (wave * NL + i) * 8 * (int)p.lda, 0, 0);
+    } else {
+      const int row = (wave >> 1) * 128 + 32 * (i & 3) + (wave & 1) * 2 + (i >> 2);
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(ld_rsB, reinterpret_cast<lds_ptr_t>(dst), 16, b_voff[i & 1] | ((i & 1) ? m_odd : m_even),
+                                               k0 + row * (int)p.ldb, 0, 0);
+    }
+  };
+
+  // ---- LDS -> register fragment plan (as in the kernel above) ----
+  const int l31 = lane & 31, h = lane >> 5;
+  const int fr = (l31 & 7) ^ ((l31 >> 3) & 1);
+  uint32_t foff[2][2];
+#pragma unroll
+  for (int s = 0; s < 2; ++s)
+#pragma unroll
+    for (int j = 0; j < 2; ++j) foff[s][j] = l31 * BK + (((s * 4 + h * 2 + j) ^ fr) * 16);
+  const int a_base = wm * (TM * 32 * BK);
+  const int b_base = wn * (TN * 32 * BK);
+  typedef const __attribute__((address_space(3))) v4i *lds_v4i_ptr;
+  auto frag_addrs = [&](int slot_a, int slot_b, int s, uint32_t (&ad)[4]) {
+    const uint32_t sa = lds0 + slot_a * UNIT + a_base, sb = lds0 + slot_b * UNIT + b_base;
+    asm volatile("v_add_u32 %0, %1, %2" : "=v"(ad[0]) : "s"(sa), "v"(foff[s][0]));
+    asm volatile("v_add_u32 %0, %1, %2" : "=v"(ad[1]) : "s"(sa), "v"(foff[s][1]));
+    asm volatile("v_add_u32 %0, %1, %2" : "=v"(ad[2]) : "s"(sb), "v"(foff[s][0]));
+    asm volatile("v_add_u32 %0, %1, %2" : "=v"(ad[3]) : "s"(sb), "v"(foff[s][1]));
+  };
+  // fragment f, in the order the MFMAs need them: A0, B0 .. B(TN-1), A1 ..
+  auto read_one = [&](const uint32_t (&ad)[4], v8i (&af)[TM], v8i (&bf)[TN], int f) {
+    const bool is_a = f == 0 || f > TN;
+    const int t = f == 0 ? 0 : (f > TN ? f - TN : f - 1);
+    const v4i lo = *reinterpret_cast<lds_v4i_ptr>(ad[is_a ? 0 : 2] + t * (32 * BK));
+    const v4i hi = *reinterpret_cast<lds_v4i_ptr>(ad[is_a ? 1 : 3] + t * (32 * BK));
+    const v8i v = v8i{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+    if (is_a) af[t] = v;
+    else bf[t] = v;
+  };
+
+  v16f acc[TM][TN];
+#pragma unroll
+  for (int tm = 0; tm < TM; ++tm)
+#pragma unroll
+    for (int tn = 0; tn < TN; ++tn)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) acc[tm][tn][v] = 0.0f;
+  // MFMA number idx of one 64-byte step, tm-major
+  auto mma_one = [&](v8i (&af)[TM], v8i (&bf)[TN], int idx) {
+    const int tm = idx / TN, tn = idx % TN;
+    acc[tm][tn] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(af[tm], bf[tn], acc[tm][tn], 0, 0, 0, 0, 0, 0);
+  };
+
+  // ---- C tile straight from the accumulators ----
+  // acc[tm][tn][4*qd + e] of lane (l31, h) is C[m][n] with m = wm*128 + tm*32 + 8*qd + 4*h + e and
+  // n = wn*128 + 4*l31 + tn (tile coordinates).  The host launches this kernel only when every lane pair's
+  // eight columns are in or out as a whole and its 16-byte store is aligned: N % 8 == 0, ldc % 8 == 0, C
+  // 16-byte aligned, row scales 16-byte and bias 8-byte aligned.
+  auto store_tile = [&](int seg) {
+    int m0, n0;
+    tile_of(seg, m0, n0);
+    // Opaque copies: everything below would otherwise be hoisted out of the K loop as loop-invariant (64 row
+    // offsets in scalar registers, per-lane addresses in vector registers) and held across it.
+    int ldc2 = (int)p.ldc * 2;
+    asm volatile("" : "+s"(ldc2));
+    int lane_col = wn * 128 + 4 * l31;
+    asm volatile("" : "+v"(lane_col));
+    {
+      const int64_t c_left = ((int64_t)(p.M - m0 - 1) * p.ldc + (p.N - n0)) * 2;
+      const __amdgpu_buffer_rsrc_t rsC = make_rsrc(p.C + (int64_t)m0 * p.ldc + n0, c_left < 0x7fffffff ? (uint32_t)c_left : 0x7fffffffu);
+      const int64_t sa_left = (int64_t)(p.M - m0) * 4, sb_left = (int64_t)(p.N - n0) * 4;
+      const __amdgpu_buffer_rsrc_t rsSa = make_rsrc(p.sa + m0, sa_left < 0x7fffffff ? (uint32_t)sa_left : 0x7fffffffu);
+      const __amdgpu_buffer_rsrc_t rsSb = make_rsrc(p.sb + n0, sb_left < 0x7fffffff ? (uint32_t)sb_left : 0x7fffffffu);
+      float sbv[4];
+      if (p.sb_row) {
+        const v4i t = __builtin_amdgcn_raw_buffer_load_b128(rsSb, lane_col * 4, 0, 0);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) sbv[e] = __int_as_float(t[e]);
+      } else {
+        const float s = p.sb[0];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) sbv[e] = s;
+      }
+      [[maybe_unused]] float bv[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+      if constexpr (HAS_BIAS) {
+        const __amdgpu_buffer_rsrc_t rsBias = make_rsrc(p.bias + n0, (uint32_t)((p.N - n0) * 2));
+        const v2i t = __builtin_amdgcn_raw_buffer_load_b64(rsBias, lane_col * 2, 0, 0);
+        bv[0] = bf16_bits_to_f32((uint32_t)t[0] & 0xffffu);
+        bv[1] = bf16_bits_to_f32((uint32_t)t[0] >> 16);
+        bv[2] = bf16_bits_to_f32((uint32_t)t[1] & 0xffffu);
+        bv[3] = bf16_bits_to_f32((uint32_t)t[1] >> 16);
+      }
+      [[maybe_unused]] uint64_t tq0 = 0, tq1 = 0, tq2 = 0;
+      if (L8_GEMM_PROF) {
+        tq0 = __builtin_readcyclecounter();
+        __builtin_amdgcn_s_waitcnt(0x0070);  // vmcnt(0), lgkmcnt(0): the panel loads in flight
+        tq1 = __builtin_readcyclecounter();
+        prof[8] += tq1 - tq0;
+      }
+      // Every scale is requested before the first store: the memory counter retires in order, so a scale load
+      // issued among the stores would make its consumer wait for all the stores ahead of it.
+      const float sa_s = p.sa[0];
+      v4i sav[TM][4];
+#pragma unroll
+      for (int tm = 0; tm < TM; ++tm)
+#pragma unroll
+        for (int qd = 0; qd < 4; ++qd) {
+          if (p.sa_row) {
+            sav[tm][qd] = __builtin_amdgcn_raw_buffer_load_b128(rsSa, h * 16, (wm * 128 + tm * 32 + 8 * qd) * 4, 0);
+          } else {
+            const int bits = __float_as_int(sa_s);
+            sav[tm][qd] = v4i{bits, bits, bits, bits};
+          }
+        }
+      // A store instruction costs the same whatever it carries, so neighbouring lanes pair up: of two
+      // consecutive rows, the even lane takes the first (its own four columns and the odd lane's four, 16
+      // contiguous bytes) and the odd lane the second.  One instruction then writes four rows x 256 bytes.
+      // Lanes whose columns lie beyond N store nothing (N % 8 == 0 here: a lane pair is in or out as a whole).
+      const int par = l31 & 1;
+      const uint32_t c_voff = (n0 + wn * 128 + 4 * (l31 & ~1) < p.N)
+                                  ? (uint32_t)((4 * h + par) * ldc2 + (lane_col - 4 * par) * 2) : kOOB;
+      if (L8_GEMM_PROF) {
+        __builtin_amdgcn_s_waitcnt(0x0070);  // the scales
+        tq2 = __builtin_readcyclecounter();
+        prof[9] += tq2 - tq1;
+      }
+#pragma unroll
+      for (int tm = 0; tm < TM; ++tm) {
+#pragma unroll
+        for (int qd = 0; qd < 4; ++qd) {
+          const int row = wm * 128 + tm * 32 + 8 * qd;  // + 4*h + e
+#pragma unroll
+          for (int e2 = 0; e2 < 4; e2 += 2) {
+            int o[2][2];  // [row e2 / e2+1][low / high pair of columns]
+#pragma unroll
+            for (int r = 0; r < 2; ++r) {
+              const float sa = __int_as_float(sav[tm][qd][e2 + r]);
+              float v[4];
+#pragma unroll
+              for (int tn = 0; tn < TN; ++tn) {
+                v[tn] = acc[tm][tn][4 * qd + e2 + r] * sa * sbv[tn];
+                if constexpr (HAS_BIAS) v[tn] += bv[tn];
+              }
+              typedef __bf16 bf2 __attribute__((ext_vector_type(2)));
+              const bf2 lo = {(__bf16)v[0], (__bf16)v[1]}, hi = {(__bf16)v[2], (__bf16)v[3]};
+              o[r][0] = __builtin_bit_cast(int, lo);
+              o[r][1] = __builtin_bit_cast(int, hi);
+            }
+            // even lanes hand over their second row, odd lanes their first; quad_perm [1,0,3,2] swaps neighbours
+            const int give0 = par ? o[0][0] : o[1][0], give1 = par ? o[0][1] : o[1][1];
+            const int got0 = __builtin_amdgcn_update_dpp(0, give0, 0xB1, 0xF, 0xF, true);
+            const int got1 = __builtin_amdgcn_update_dpp(0, give1, 0xB1, 0xF, 0xF, true);
+            const v4i out = par ? v4i{got0, got1, o[1][0], o[1][1]} : v4i{o[0][0], o[0][1], got0, got1};
+            __builtin_amdgcn_raw_buffer_store_b128(out, rsC, c_voff, (row + e2) * ldc2, 2 /* streaming */);
+          }
+        }
+      }
+      if (L8_GEMM_PROF) {
+        tq0 = __builtin_readcyclecounter();
+        prof[10] += tq0 - tq2;
+        __builtin_amdgcn_s_waitcnt(0x0070);  // the stores
+        prof[11] += __builtin_readcyclecounter() - tq0;
+      }
+    }
+#pragma unroll
+    for (int tm = 0; tm < TM; ++tm)
+#pragma unroll
+      for (int tn = 0; tn < TN; ++tn)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) acc[tm][tn][v] = 0.0f;
+  };
+
+  if (L8_GEMM_PROF) {
+    prof[0] = __builtin_amdgcn_s_memrealtime();
+    prof[5] = __builtin_readcyclecounter();
+  }
+  if (L8_GEMM_DIAG == 5 || L8_GEMM_DIAG == 6) {  // experiments: XCD x starts x/8 of a tile's duration late (5); workgroup loc of an XCD starts loc/256 of it late (6)
+    const uint64_t t_go = __builtin_amdgcn_s_memrealtime() + (L8_GEMM_DIAG == 5 ? (uint64_t)xcd * (uint64_t)KT * 17 : (uint64_t)loc * (uint64_t)KT * 17 / 32);  // ~1.36 us per K tile, 100 MHz ticks
+    while (__builtin_amdgcn_s_memrealtime() < t_go) __builtin_amdgcn_s_sleep(8);
+  }
+  // ---- prologue: K tiles 0 and 1 of the workgroup's stream requested, K tile 0 published, its first step read ----
+  ld_open(0);
+#pragma unroll
+  for (int u = 0; u < R - 1; ++u) {
+#pragma unroll
+    for (int i = 0; i < NL; ++i) load_one(u & 1, u, i);
+    if (u & 1) ld_advance();
+  }
+  v8i af0[TM], bf0[TN], af1[TM], bf1[TN];
+  uint32_t ad[4];
+  L8_WAIT_VM_LGKM0(PEND0);
+  asm volatile("" ::: "memory");
+  __builtin_amdgcn_s_barrier();
+  asm volatile("" ::: "memory");
+  frag_addrs(0, 1, 0, ad);
+#pragma unroll
+  for (int f = 0; f < TM + TN; ++f) read_one(ad, af0, bf0, f);
+
+  // One trip = one K tile = two matrix-core steps of 64, laid out as in the kernel above: first half = MFMAs
+  // of step 0 + LDS reads of step 1 + requests for the A panel two K tiles ahead; barrier; second half =
+  // MFMAs of step 1 + LDS reads of the next K tile's step 0 + requests for the matching B panel.
+  constexpr int N_MMA = TM * TN, NF = TM + TN;
+  constexpr int STRADDLE = L8_STRADDLE < N_MMA - 2 ? L8_STRADDLE : 0;
+  constexpr int S1 = N_MMA - STRADDLE, S2 = N_MMA + STRADDLE, SR = N_MMA - 2;
+  int s0 = 0;  // ring slot of the A panel of the K tile being multiplied
+#pragma unroll 1
+  for (int seg = 0; seg < n_seg; ++seg) {
+    // Everything older than the NL loads just requested must have landed at the barrier of a trip.  In the first
+    // trip after the N_STORES stores of a C tile (younger than the panels needed there) the count allows for
+    // them: the counter retires in order, and waiting for the stores themselves would stall every tile's start.
+    bool after_store = seg > 0;
+    [[maybe_unused]] uint64_t t_loop = 0;
+    if (L8_GEMM_PROF) {
+      if (seg == 0) prof[1] = __builtin_amdgcn_s_memrealtime();
+      t_loop = __builtin_readcyclecounter();
+    }
+#pragma unroll 1
+    for (int kt = 0; kt < KT; ++kt) {
+      const int slot_u1 = wrap(s0 + R - 1);
+      frag_addrs(s0, wrap(s0 + 1), 1, ad);
+#pragma unroll
+      for (int i = 0; i < S1; ++i) {
+        mma_one(af0, bf0, i);
+#pragma unroll
+        for (int f = (NF * i) / S1; f < (NF * (i + 1)) / S1; ++f) read_one(ad, af1, bf1, f);
+#pragma unroll
+        for (int j = (NL * i) / S1; j < (NL * (i + 1)) / S1; ++j) load_one(false, slot_u1, j);
+        __builtin_amdgcn_sched_barrier(0);
+      }
+      if (after_store) L8_WAIT_VM_LGKM0(N_STORES + PEND);
+      else L8_WAIT_VM_LGKM0(PEND);
+      after_store = false;
+      asm volatile("" ::: "memory");
+      __builtin_amdgcn_s_barrier();
+      asm volatile("" ::: "memory");
+      frag_addrs(wrap(s0 + 2), wrap(s0 + 3), 0, ad);
+#pragma unroll
+      for (int i = 0; i < S2; ++i) {
+        if (i < STRADDLE) mma_one(af0, bf0, S1 + i);
+        else mma_one(af1, bf1, i - STRADDLE);
+        if (i >= STRADDLE) {
+#pragma unroll
+          for (int f = (NF * (i - STRADDLE)) / SR; f < (NF * (i - STRADDLE + 1)) / SR && f < NF; ++f) read_one(ad, af0, bf0, f);
+        }
+#pragma unroll
+        for (int j = (NL * i) / S2; j < (NL * (i + 1)) / S2; ++j) load_one(true, s0, j);
+        __builtin_amdgcn_sched_barrier(0);
+      }
+      ld_advance();
+      s0 = wrap(s0 + 2);
+    }
+    if (L8_GEMM_PROF) {
+      const uint64_t t = __builtin_readcyclecounter();
+      prof[3] += t - t_loop;
+      t_loop = t;
+    }
+    store_tile(seg);
+    if (L8_GEMM_PROF) prof[4] += __builtin_readcyclecounter() - t_loop;
+  }
+  // the tail requests (out of range, zero filling) must have landed before the workgroup's LDS is released
+  L8_WAIT_VM_LGKM0(0);
+  if (L8_GEMM_PROF) {
+    prof[2] = __builtin_amdgcn_s_memrealtime();
+    prof[5] = __builtin_readcyclecounter() - prof[5];
+    prof[6] = n_seg;
+    prof[7] = ((uint64_t)__builtin_amdgcn_s_getreg(63508) << 32) | (uint32_t)__builtin_amdgcn_s_getreg(63492);  // XCC_ID, HW_ID
+    if (threadIdx.x == 0 && p.dbg) {
+      uint64_t *d = p.dbg + (int64_t)blockIdx.x * 16;
+      for (int i = 0; i < 16; ++i) d[i] = prof[i];
+    }
+  }
+#else
+  (void)p;
+#endif
+}
+
+// ---------------------------------------------------------------------------
 // tile configurations ("algos")
 // ---------------------------------------------------------------------------
 typedef void (*gemm_fn)(const GemmArgs);
@@ -483,6 +864,8 @@ struct Algo {
   const char *name;
   gemm_fn fn;
   int bm, bn, threads, lds;
+  bool persistent;   // one workgroup per compute unit walks a list of tiles
+  gemm_fn fn_bias;   // persistent kernels: the instantiation that adds a bias (the plain kernels branch inside)
 };
 
 // X(WM, WN, TM, TN, R, GROUP_M, PF) -- 1-based position in this list is the `algo` number
@@ -505,9 +888,19 @@ L8_ALGO_LIST(L8_INSTANTIATE)
 #define L8_MAX2(a, b) ((a) > (b) ? (a) : (b))
 #define L8_ALGO_ROW(WM, WN, TM, TN, R, GM, PF)                                                                \
   {"mt" #WM "x" #WN "w_" #TM "x" #TN "t_r" #R "_g" #GM "_pf" #PF, gemm_nt_kernel<WM, WN, TM, TN, R, GM, PF>, \
-   WM * TM * 32, WN * TN * 32, WM * WN * 64, R * L8_MAX2(WM * TM * 32, WN * TN * 32) * 128},
+   WM * TM * 32, WN * TN * 32, WM * WN * 64, R * L8_MAX2(WM * TM * 32, WN * TN * 32) * 128, false, nullptr},
 
-static const Algo kAlgos[] = {L8_ALGO_LIST(L8_ALGO_ROW)};
+template __global__ void gemm_nt_stream_kernel<8, false>(const GemmArgs);
+template __global__ void gemm_nt_stream_kernel<8, true>(const GemmArgs);
+template __global__ void gemm_nt_stream_kernel<4, false>(const GemmArgs);
+template __global__ void gemm_nt_stream_kernel<4, true>(const GemmArgs);
+
+static const Algo kAlgos[] = {
+    L8_ALGO_LIST(L8_ALGO_ROW)
+    /* 11, 12: persistent 256x256 tiles, 4 waves, one panel stream across tiles, C stored from the accumulators */
+    {"stream_mt2x2w_4x4t_r5_g8", gemm_nt_stream_kernel<8, false>, 256, 256, 256, 5 * 256 * 128, true, gemm_nt_stream_kernel<8, true>},
+    {"stream_mt2x2w_4x4t_r5_g4", gemm_nt_stream_kernel<4, false>, 256, 256, 256, 5 * 256 * 128, true, gemm_nt_stream_kernel<4, true>},
+};
 constexpr int kNumAlgos = sizeof(kAlgos) / sizeof(kAlgos[0]);
 
 }  // namespace l8
@@ -547,6 +940,14 @@ extern "C" int l8_gemm_nt(const void *A, const void *B, int64_t M, int64_t N, in
   L8_REQUIRE(M < (1LL << 31) && N < (1LL << 31) && K < (1LL << 31), "l8_gemm_nt: dimension too large");
   L8_REQUIRE(algo >= 0 && algo <= kNumAlgos, "l8_gemm_nt: algo %d out of range 0..%d", algo, kNumAlgos);
   if (algo == 0) algo = pick_algo(M, N, K);
+  if (kAlgos[algo - 1].persistent) {
+    // the persistent kernel stores 16 aligned bytes (eight columns) per lane and reads the row scales 16 bytes
+    // at a time; operands that do not allow that go to the plain kernel with the same tile shape
+    const bool ok = N % 8 == 0 && ldc % 8 == 0 && ((uintptr_t)C % 16) == 0 && ldc < (1LL << 22) &&
+                    (sa_mode != L8_SCALE_ROW || ((uintptr_t)sa % 16) == 0) &&
+                    (sb_mode != L8_SCALE_ROW || ((uintptr_t)sb % 16) == 0) && (bias == nullptr || ((uintptr_t)bias % 8) == 0);
+    if (!ok) algo = 5;
+  }
   const Algo &al = kAlgos[algo - 1];
   // 32-bit in-tile byte offsets: (tile rows) * ld + K must stay below 2^31
   L8_REQUIRE((int64_t)al.bm * lda + K < (1LL << 31) && (int64_t)al.bn * ldb + K < (1LL << 31),
@@ -565,6 +966,11 @@ extern "C" int l8_gemm_nt(const void *A, const void *B, int64_t M, int64_t N, in
   p.sa_row = sa_mode == L8_SCALE_ROW;
   p.sb_row = sb_mode == L8_SCALE_ROW;
   p.bias = (const uint16_t *)bias;
+  p.dbg = nullptr;
+  if (L8_GEMM_PROF && al.persistent) {
+    p.dbg = (uint64_t *)bias;
+    p.bias = nullptr;
+  }
   p.C = (uint16_t *)C;
   p.tiles_m = (int)((M + al.bm - 1) / al.bm);
   p.tiles_n = (int)((N + al.bn - 1) / al.bn);
@@ -574,9 +980,19 @@ extern "C" int l8_gemm_nt(const void *A, const void *B, int64_t M, int64_t N, in
   const int slot = device_slot();
   if (slot < 0 || !attr_done[slot][algo - 1]) {
     L8_HIP(hipFuncSetAttribute((const void *)al.fn, hipFuncAttributeMaxDynamicSharedMemorySize, al.lds));
+    if (al.fn_bias) L8_HIP(hipFuncSetAttribute((const void *)al.fn_bias, hipFuncAttributeMaxDynamicSharedMemorySize, al.lds));
     if (slot >= 0) attr_done[slot][algo - 1] = true;
   }
-  hipLaunchKernelGGL(al.fn, dim3((unsigned)nblocks), dim3(al.threads), al.lds, (hipStream_t)stream, p);
+  int64_t grid = nblocks;
+  if (al.persistent) {
+    // one workgroup per compute unit, a multiple of 8 of them (the hardware deals workgroups to the 8 XCDs in turn)
+    const int64_t cus8 = (num_cus() / 8) * 8;
+    const int64_t want = (nblocks + 7) / 8 * 8;
+    grid = want < cus8 ? want : cus8;
+    if (grid < 8) grid = 8;
+  }
+  const gemm_fn fn = (al.fn_bias && p.bias) ? al.fn_bias : al.fn;
+  hipLaunchKernelGGL(fn, dim3((unsigned)grid), dim3(al.threads), al.lds, (hipStream_t)stream, p);
   L8_HIP(hipGetLastError());
   return L8_OK;
 }

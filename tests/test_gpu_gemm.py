@@ -21,7 +21,7 @@ def fp8(t):
     return t.to(torch.float8_e4m3fn)
 
 
-ALGOS = list(range(0, 10))
+ALGOS = list(range(0, 13))
 SHAPES_EXACT = [(1, 1, 16), (32, 32, 64), (256, 256, 128), (256, 256, 256), (300, 200, 144), (257, 513, 272),
                 (64, 1000, 48), (1000, 24, 208), (512, 768, 240)]
 
@@ -42,7 +42,7 @@ def test_exact_small_integer_operands(algo):
         assert torch.equal(out.cpu().double(), want), (algo, M, N, K)
 
 
-@pytest.mark.parametrize("algo", [0, 1, 2, 3])
+@pytest.mark.parametrize("algo", [0, 1, 2, 3, 11])
 def test_k_indexing_with_one_hot_operands(algo):
     # B[n] is one-hot at k = pi(n): C[m,n] = A[m, pi(n)] exactly, for any K (tails included)
     from lingua_amd import ops
