@@ -638,111 +638,136 @@ __global__ __launch_bounds__(256) void gemm_nt_stream_kernel(const GemmArgs p) {
   // n = wn*128 + 4*l31 + tn (tile coordinates).  The host launches this kernel only when every lane pair's
   // eight columns are in or out as a whole and its 16-byte store is aligned: N % 8 == 0, ldc % 8 == 0, C
   // 16-byte aligned, row scales 16-byte and bias 8-byte aligned.
+  // The scales (and the bias) of a tile are requested before its K loop, a handful of registers per lane: lane l
+  // holds the A scales of tile rows wm*128 + l and + 64 + l (handed to the lanes that need them by lane
+  // permutes at the end) and the B scales / bias of its own four columns.  Requested among the stores of the
+  // tile they would make their consumer wait for every store ahead of them (the counter retires in order).
+  int seg_sa[2] = {0, 0};
+  v4i seg_sb = {0, 0, 0, 0};
+  [[maybe_unused]] v2i seg_bias = {0, 0};
+  auto load_scales = [&](int seg) {
+    int m0, n0;
+    tile_of(seg, m0, n0);
+    const int64_t sa_left = (int64_t)(p.M - m0) * 4, sb_left = (int64_t)(p.N - n0) * 4;
+    if (p.sa_row) {
+      const __amdgpu_buffer_rsrc_t rsSa = make_rsrc(p.sa + m0, sa_left < 0x7fffffff ? (uint32_t)sa_left : 0x7fffffffu);
+      seg_sa[0] = __builtin_amdgcn_raw_buffer_load_b32(rsSa, (wm * 128 + lane) * 4, 0, 0);
+      seg_sa[1] = __builtin_amdgcn_raw_buffer_load_b32(rsSa, (wm * 128 + 64 + lane) * 4, 0, 0);
+    } else {
+      seg_sa[0] = seg_sa[1] = __float_as_int(p.sa[0]);
+    }
+    if (p.sb_row) {
+      const __amdgpu_buffer_rsrc_t rsSb = make_rsrc(p.sb + n0, sb_left < 0x7fffffff ? (uint32_t)sb_left : 0x7fffffffu);
+      seg_sb = __builtin_amdgcn_raw_buffer_load_b128(rsSb, (wn * 128 + 4 * l31) * 4, 0, 0);
+    } else {
+      const int bits = __float_as_int(p.sb[0]);
+      seg_sb = v4i{bits, bits, bits, bits};
+    }
+    if constexpr (HAS_BIAS) {
+      const __amdgpu_buffer_rsrc_t rsBias = make_rsrc(p.bias + n0, (uint32_t)((p.N - n0) * 2));
+      seg_bias = __builtin_amdgcn_raw_buffer_load_b64(rsBias, (wn * 128 + 4 * l31) * 2, 0, 0);
+    }
+  };
+  // (A compute unit drains its stores at about 16 bytes per clock: the 128 KiB of a C tile keep it busy for some
+  // 8000 cycles, of which the conversion below hides about half.)
   auto store_tile = [&](int seg) {
     int m0, n0;
     tile_of(seg, m0, n0);
-    // Opaque copies: everything below would otherwise be hoisted out of the K loop as loop-invariant (64 row
+    // Opaque copies: everything below would otherwise be hoisted out of the K loop as loop-invariant (row
     // offsets in scalar registers, per-lane addresses in vector registers) and held across it.
     int ldc2 = (int)p.ldc * 2;
     asm volatile("" : "+s"(ldc2));
     int lane_col = wn * 128 + 4 * l31;
     asm volatile("" : "+v"(lane_col));
-    {
-      const int64_t c_left = ((int64_t)(p.M - m0 - 1) * p.ldc + (p.N - n0)) * 2;
-      const __amdgpu_buffer_rsrc_t rsC = make_rsrc(p.C + (int64_t)m0 * p.ldc + n0, c_left < 0x7fffffff ? (uint32_t)c_left : 0x7fffffffu);
-      const int64_t sa_left = (int64_t)(p.M - m0) * 4, sb_left = (int64_t)(p.N - n0) * 4;
-      const __amdgpu_buffer_rsrc_t rsSa = make_rsrc(p.sa + m0, sa_left < 0x7fffffff ? (uint32_t)sa_left : 0x7fffffffu);
-      const __amdgpu_buffer_rsrc_t rsSb = make_rsrc(p.sb + n0, sb_left < 0x7fffffff ? (uint32_t)sb_left : 0x7fffffffu);
-      float sbv[4];
-      if (p.sb_row) {
-        const v4i t = __builtin_amdgcn_raw_buffer_load_b128(rsSb, lane_col * 4, 0, 0);
+    const int64_t c_left = ((int64_t)(p.M - m0 - 1) * p.ldc + (p.N - n0)) * 2;
+    const __amdgpu_buffer_rsrc_t rsC = make_rsrc(p.C + (int64_t)m0 * p.ldc + n0, c_left < 0x7fffffff ? (uint32_t)c_left : 0x7fffffffu);
+    float sbv[4];
+    [[maybe_unused]] float bv[4];
 #pragma unroll
-        for (int e = 0; e < 4; ++e) sbv[e] = __int_as_float(t[e]);
-      } else {
-        const float s = p.sb[0];
+    for (int e = 0; e < 4; ++e) sbv[e] = __int_as_float(seg_sb[e]);
+    if constexpr (HAS_BIAS) {
+      bv[0] = bf16_bits_to_f32((uint32_t)seg_bias[0] & 0xffffu);
+      bv[1] = bf16_bits_to_f32((uint32_t)seg_bias[0] >> 16);
+      bv[2] = bf16_bits_to_f32((uint32_t)seg_bias[1] & 0xffffu);
+      bv[3] = bf16_bits_to_f32((uint32_t)seg_bias[1] >> 16);
+    }
+    // Row scale of tile row wm*128 + r: lane r % 64 of seg_sa[r / 64]; a lane needs r = tm*32 + 8*qd + 4*h + e.
+    // The lane permutes of the next (tm, qd) group are in flight while the current group is converted.  They are
+    // written as assembly for the immediate offset (as plain address arithmetic the 64 addresses were
+    // precomputed into 64 registers and spilled) and are waited for by hand: LDS operations return in order, so
+    // "at most 4 outstanding" means that everything but the group requested last has arrived.
+    const int sa_addr = 16 * h;  // byte address of lane 4*h
+    float sa_grp[2][4];
+    auto request_row_scales = [&](int g, float (&dst)[4]) {  // g = tm * 4 + qd
+      const int tm = g >> 2, qd = g & 3;
 #pragma unroll
-        for (int e = 0; e < 4; ++e) sbv[e] = s;
-      }
-      [[maybe_unused]] float bv[4] = {0.0f, 0.0f, 0.0f, 0.0f};
-      if constexpr (HAS_BIAS) {
-        const __amdgpu_buffer_rsrc_t rsBias = make_rsrc(p.bias + n0, (uint32_t)((p.N - n0) * 2));
-        const v2i t = __builtin_amdgcn_raw_buffer_load_b64(rsBias, lane_col * 2, 0, 0);
-        bv[0] = bf16_bits_to_f32((uint32_t)t[0] & 0xffffu);
-        bv[1] = bf16_bits_to_f32((uint32_t)t[0] >> 16);
-        bv[2] = bf16_bits_to_f32((uint32_t)t[1] & 0xffffu);
-        bv[3] = bf16_bits_to_f32((uint32_t)t[1] >> 16);
-      }
-      [[maybe_unused]] uint64_t tq0 = 0, tq1 = 0, tq2 = 0;
-      if (L8_GEMM_PROF) {
-        tq0 = __builtin_readcyclecounter();
-        __builtin_amdgcn_s_waitcnt(0x0070);  // vmcnt(0), lgkmcnt(0): the panel loads in flight
-        tq1 = __builtin_readcyclecounter();
-        prof[8] += tq1 - tq0;
-      }
-      // Every scale is requested before the first store: the memory counter retires in order, so a scale load
-      // issued among the stores would make its consumer wait for all the stores ahead of it.
-      const float sa_s = p.sa[0];
-      v4i sav[TM][4];
+      for (int e = 0; e < 4; ++e)
+        asm volatile("ds_bpermute_b32 %0, %1, %2 offset:%3"
+                     : "=v"(dst[e])
+                     : "v"(sa_addr), "v"(seg_sa[tm >> 1]), "n"(4 * ((tm & 1) * 32 + 8 * qd + e)));
+    };
+    request_row_scales(0, sa_grp[0]);
+    [[maybe_unused]] uint64_t tq0 = 0, tq1 = 0, tq2 = 0;
+    if (L8_GEMM_PROF) {
+      tq0 = __builtin_readcyclecounter();
+      __builtin_amdgcn_s_waitcnt(0x0070);  // vmcnt(0), lgkmcnt(0): the panel loads in flight
+      tq1 = __builtin_readcyclecounter();
+      prof[8] += tq1 - tq0;
+    }
+    // A store instruction costs the same whatever it carries, so neighbouring lanes pair up: of two consecutive
+    // rows, the even lane takes the first (its own four columns and the odd lane's four, 16 contiguous bytes)
+    // and the odd lane the second.  One instruction then writes four rows x 256 bytes.  Lanes whose columns lie
+    // beyond N store nothing (N % 8 == 0 here: a lane pair is in or out as a whole).
+    const int par = l31 & 1;
+    const uint32_t c_voff = (n0 + wn * 128 + 4 * (l31 & ~1) < p.N)
+                                ? (uint32_t)((4 * h + par) * ldc2 + (lane_col - 4 * par) * 2) : kOOB;
+    if (L8_GEMM_PROF) {
+      __builtin_amdgcn_s_waitcnt(0x0070);  // the scales
+      tq2 = __builtin_readcyclecounter();
+      prof[9] += tq2 - tq1;
+    }
 #pragma unroll
-      for (int tm = 0; tm < TM; ++tm)
+    for (int tm = 0; tm < TM; ++tm) {
 #pragma unroll
-        for (int qd = 0; qd < 4; ++qd) {
-          if (p.sa_row) {
-            sav[tm][qd] = __builtin_amdgcn_raw_buffer_load_b128(rsSa, h * 16, (wm * 128 + tm * 32 + 8 * qd) * 4, 0);
-          } else {
-            const int bits = __float_as_int(sa_s);
-            sav[tm][qd] = v4i{bits, bits, bits, bits};
-          }
+      for (int qd = 0; qd < 4; ++qd) {
+        const int row = wm * 128 + tm * 32 + 8 * qd;  // + 4*h + e
+        const int g = tm * 4 + qd;
+        float(&sa_cur)[4] = sa_grp[g & 1];
+        if (g + 1 < TM * 4) {
+          request_row_scales(g + 1, sa_grp[(g + 1) & 1]);
+          asm volatile("s_waitcnt lgkmcnt(4)" : "+v"(sa_cur[0]), "+v"(sa_cur[1]), "+v"(sa_cur[2]), "+v"(sa_cur[3]));
+        } else {
+          asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(sa_cur[0]), "+v"(sa_cur[1]), "+v"(sa_cur[2]), "+v"(sa_cur[3]));
         }
-      // A store instruction costs the same whatever it carries, so neighbouring lanes pair up: of two
-      // consecutive rows, the even lane takes the first (its own four columns and the odd lane's four, 16
-      // contiguous bytes) and the odd lane the second.  One instruction then writes four rows x 256 bytes.
-      // Lanes whose columns lie beyond N store nothing (N % 8 == 0 here: a lane pair is in or out as a whole).
-      const int par = l31 & 1;
-      const uint32_t c_voff = (n0 + wn * 128 + 4 * (l31 & ~1) < p.N)
-                                  ? (uint32_t)((4 * h + par) * ldc2 + (lane_col - 4 * par) * 2) : kOOB;
-      if (L8_GEMM_PROF) {
-        __builtin_amdgcn_s_waitcnt(0x0070);  // the scales
-        tq2 = __builtin_readcyclecounter();
-        prof[9] += tq2 - tq1;
-      }
 #pragma unroll
-      for (int tm = 0; tm < TM; ++tm) {
+        for (int e2 = 0; e2 < 4; e2 += 2) {
+          int o[2][2];  // [row e2 / e2+1][low / high pair of columns]
 #pragma unroll
-        for (int qd = 0; qd < 4; ++qd) {
-          const int row = wm * 128 + tm * 32 + 8 * qd;  // + 4*h + e
+          for (int r = 0; r < 2; ++r) {
+            const float sa = sa_cur[e2 + r];
+            float v[4];
 #pragma unroll
-          for (int e2 = 0; e2 < 4; e2 += 2) {
-            int o[2][2];  // [row e2 / e2+1][low / high pair of columns]
-#pragma unroll
-            for (int r = 0; r < 2; ++r) {
-              const float sa = __int_as_float(sav[tm][qd][e2 + r]);
-              float v[4];
-#pragma unroll
-              for (int tn = 0; tn < TN; ++tn) {
-                v[tn] = acc[tm][tn][4 * qd + e2 + r] * sa * sbv[tn];
-                if constexpr (HAS_BIAS) v[tn] += bv[tn];
-              }
-              typedef __bf16 bf2 __attribute__((ext_vector_type(2)));
-              const bf2 lo = {(__bf16)v[0], (__bf16)v[1]}, hi = {(__bf16)v[2], (__bf16)v[3]};
-              o[r][0] = __builtin_bit_cast(int, lo);
-              o[r][1] = __builtin_bit_cast(int, hi);
+            for (int tn = 0; tn < TN; ++tn) {
+              v[tn] = acc[tm][tn][4 * qd + e2 + r] * sa * sbv[tn];
+              if constexpr (HAS_BIAS) v[tn] += bv[tn];
             }
-            // even lanes hand over their second row, odd lanes their first; quad_perm [1,0,3,2] swaps neighbours
-            const int give0 = par ? o[0][0] : o[1][0], give1 = par ? o[0][1] : o[1][1];
-            const int got0 = __builtin_amdgcn_update_dpp(0, give0, 0xB1, 0xF, 0xF, true);
-            const int got1 = __builtin_amdgcn_update_dpp(0, give1, 0xB1, 0xF, 0xF, true);
-            const v4i out = par ? v4i{got0, got1, o[1][0], o[1][1]} : v4i{o[0][0], o[0][1], got0, got1};
-            __builtin_amdgcn_raw_buffer_store_b128(out, rsC, c_voff, (row + e2) * ldc2, 2 /* streaming */);
+            typedef __bf16 bf2 __attribute__((ext_vector_type(2)));
+            const bf2 lo = {(__bf16)v[0], (__bf16)v[1]}, hi = {(__bf16)v[2], (__bf16)v[3]};
+            o[r][0] = __builtin_bit_cast(int, lo);
+            o[r][1] = __builtin_bit_cast(int, hi);
           }
+          // even lanes hand over their second row, odd lanes their first; quad_perm [1,0,3,2] swaps neighbours
+          const int give0 = par ? o[0][0] : o[1][0], give1 = par ? o[0][1] : o[1][1];
+          const int got0 = __builtin_amdgcn_update_dpp(0, give0, 0xB1, 0xF, 0xF, true);
+          const int got1 = __builtin_amdgcn_update_dpp(0, give1, 0xB1, 0xF, 0xF, true);
+          const v4i out = par ? v4i{got0, got1, o[1][0], o[1][1]} : v4i{o[0][0], o[0][1], got0, got1};
+          __builtin_amdgcn_raw_buffer_store_b128(out, rsC, c_voff, (row + e2) * ldc2, 2 /* streaming */);
         }
       }
-      if (L8_GEMM_PROF) {
-        tq0 = __builtin_readcyclecounter();
-        prof[10] += tq0 - tq2;
-        __builtin_amdgcn_s_waitcnt(0x0070);  // the stores
-        prof[11] += __builtin_readcyclecounter() - tq0;
-      }
+    }
+    if (L8_GEMM_PROF) {
+      tq0 = __builtin_readcyclecounter();
+      prof[10] += tq0 - tq2;
     }
 #pragma unroll
     for (int tm = 0; tm < TM; ++tm)
@@ -752,10 +777,6 @@ __global__ __launch_bounds__(256) void gemm_nt_stream_kernel(const GemmArgs p) {
         for (int v = 0; v < 16; ++v) acc[tm][tn][v] = 0.0f;
   };
 
-  if (L8_GEMM_PROF) {
-    prof[0] = __builtin_amdgcn_s_memrealtime();
-    prof[5] = __builtin_readcyclecounter();
-  }
   if (L8_GEMM_DIAG == 5 || L8_GEMM_DIAG == 6) {  // experiments: XCD x starts x/8 of a tile's duration late (5); workgroup loc of an XCD starts loc/256 of it late (6)
     const uint64_t t_go = __builtin_amdgcn_s_memrealtime() + (L8_GEMM_DIAG == 5 ? (uint64_t)xcd * (uint64_t)KT * 17 : (uint64_t)loc * (uint64_t)KT * 17 / 32);  // ~1.36 us per K tile, 100 MHz ticks
     while (__builtin_amdgcn_s_memrealtime() < t_go) __builtin_amdgcn_s_sleep(8);
@@ -785,52 +806,60 @@ __global__ __launch_bounds__(256) void gemm_nt_stream_kernel(const GemmArgs p) {
   constexpr int STRADDLE = L8_STRADDLE < N_MMA - 2 ? L8_STRADDLE : 0;
   constexpr int S1 = N_MMA - STRADDLE, S2 = N_MMA + STRADDLE, SR = N_MMA - 2;
   int s0 = 0;  // ring slot of the A panel of the K tile being multiplied
+  // WAIT = the count of the wait in front of the barrier: everything older than the WAIT youngest requests must
+  // have landed.
+  auto trip = [&](auto wait_tag) {
+    constexpr int WAIT = decltype(wait_tag)::value;
+    const int slot_u1 = wrap(s0 + R - 1);
+    frag_addrs(s0, wrap(s0 + 1), 1, ad);
+#pragma unroll
+    for (int i = 0; i < S1; ++i) {
+      mma_one(af0, bf0, i);
+#pragma unroll
+      for (int f = (NF * i) / S1; f < (NF * (i + 1)) / S1; ++f) read_one(ad, af1, bf1, f);
+#pragma unroll
+      for (int j = (NL * i) / S1; j < (NL * (i + 1)) / S1; ++j) load_one(false, slot_u1, j);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    L8_WAIT_VM_LGKM0(WAIT);
+    asm volatile("" ::: "memory");
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
+    frag_addrs(wrap(s0 + 2), wrap(s0 + 3), 0, ad);
+#pragma unroll
+    for (int i = 0; i < S2; ++i) {
+      if (i < STRADDLE) mma_one(af0, bf0, S1 + i);
+      else mma_one(af1, bf1, i - STRADDLE);
+      if (i >= STRADDLE) {
+#pragma unroll
+        for (int f = (NF * (i - STRADDLE)) / SR; f < (NF * (i - STRADDLE + 1)) / SR && f < NF; ++f) read_one(ad, af0, bf0, f);
+      }
+#pragma unroll
+      for (int j = (NL * i) / S2; j < (NL * (i + 1)) / S2; ++j) load_one(true, s0, j);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    ld_advance();
+    s0 = wrap(s0 + 2);
+  };
+  using std::integral_constant;
 #pragma unroll 1
   for (int seg = 0; seg < n_seg; ++seg) {
-    // Everything older than the NL loads just requested must have landed at the barrier of a trip.  In the first
-    // trip after the N_STORES stores of a C tile (younger than the panels needed there) the count allows for
-    // them: the counter retires in order, and waiting for the stores themselves would stall every tile's start.
-    bool after_store = seg > 0;
     [[maybe_unused]] uint64_t t_loop = 0;
     if (L8_GEMM_PROF) {
       if (seg == 0) prof[1] = __builtin_amdgcn_s_memrealtime();
       t_loop = __builtin_readcyclecounter();
     }
-#pragma unroll 1
-    for (int kt = 0; kt < KT; ++kt) {
-      const int slot_u1 = wrap(s0 + R - 1);
-      frag_addrs(s0, wrap(s0 + 1), 1, ad);
-#pragma unroll
-      for (int i = 0; i < S1; ++i) {
-        mma_one(af0, bf0, i);
-#pragma unroll
-        for (int f = (NF * i) / S1; f < (NF * (i + 1)) / S1; ++f) read_one(ad, af1, bf1, f);
-#pragma unroll
-        for (int j = (NL * i) / S1; j < (NL * (i + 1)) / S1; ++j) load_one(false, slot_u1, j);
-        __builtin_amdgcn_sched_barrier(0);
-      }
-      if (after_store) L8_WAIT_VM_LGKM0(N_STORES + PEND);
-      else L8_WAIT_VM_LGKM0(PEND);
-      after_store = false;
-      asm volatile("" ::: "memory");
-      __builtin_amdgcn_s_barrier();
-      asm volatile("" ::: "memory");
-      frag_addrs(wrap(s0 + 2), wrap(s0 + 3), 0, ad);
-#pragma unroll
-      for (int i = 0; i < S2; ++i) {
-        if (i < STRADDLE) mma_one(af0, bf0, S1 + i);
-        else mma_one(af1, bf1, i - STRADDLE);
-        if (i >= STRADDLE) {
-#pragma unroll
-          for (int f = (NF * (i - STRADDLE)) / SR; f < (NF * (i - STRADDLE + 1)) / SR && f < NF; ++f) read_one(ad, af0, bf0, f);
-        }
-#pragma unroll
-        for (int j = (NL * i) / S2; j < (NL * (i + 1)) / S2; ++j) load_one(true, s0, j);
-        __builtin_amdgcn_sched_barrier(0);
-      }
-      ld_advance();
-      s0 = wrap(s0 + 2);
+    load_scales(seg);
+    int kt = 0;
+    if (seg > 0) {
+      // The first barrier after the N_STORES stores of a C tile: they are younger than the panels waited for
+      // and the counter retires in order, so the count allows for them (waiting for the stores themselves would
+      // stall the start of every tile).
+      trip(integral_constant<int, N_STORES + PEND>{});
+      kt = 1;
     }
+#pragma unroll 1
+    for (; kt < KT; ++kt) trip(integral_constant<int, PEND>{});
     if (L8_GEMM_PROF) {
       const uint64_t t = __builtin_readcyclecounter();
       prof[3] += t - t_loop;
