@@ -10,7 +10,9 @@ MLP = 9 GEMMs of 2*16384*4096*11008 flop = 13 297 218 748 416 flop.
 Prints ONE JSON line.  `value` is TFLOP/s over whole steps (casts, SiLU and
 autograd bookkeeping included) with inputs resident in HBM.  `roofline` is the
 GEMM kernel alone, timed with events on its stream inside the timed steps.
-`cpu_baseline` is the same recipe as PyTorch CPU ops on a token sample.
+`cpu_baseline` is the same recipe as PyTorch CPU ops on a token sample.  `sustained` is the same step run for
+two seconds; `extras` holds side measurements (never part of `value`): the fused-gate path, torch._scaled_mm on
+the step's GEMM shapes, one Fp8Linear forward+backward, the config-4 figures and the Llama-1B-shaped step.
 """
 import argparse
 import json
@@ -48,8 +50,11 @@ def parse():
                          "tokens (casts included); llama1b = full Llama-1B-shaped forward+backward step "
                          "(25 layers, dim 2048, ffn 8192, vocab 128256, 4 x 4096 tokens), reported in tokens/s")
     ap.add_argument("--no-extras", action="store_true",
-                    help="skip the two side measurements: the fused-SwiGLU variant of the same MLP and "
-                         "torch._scaled_mm (what the reference calls) on the step's GEMM shapes")
+                    help="skip the side measurements: the sustained leg, the fused-SwiGLU variant of the same MLP, "
+                         "torch._scaled_mm (what the reference calls) on the step's GEMM shapes, one Fp8Linear, the "
+                         "config-4 figures and the Llama-1B step")
+    ap.add_argument("--sustained-seconds", type=float, default=2.0,
+                    help="length of the sustained leg (same step, run for at least this long)")
     ap.add_argument("--gemm-shape", choices=["fwd", "dgrad", "wgrad"], default="fwd",
                     help="with --kernel-only gemm: which product of the 4096 -> 11008 linear (reduction 4096, 11008, 16384)")
     ap.add_argument("--launches", type=int, default=3, help="with --kernel-only gemm: number of launches")
@@ -100,6 +105,15 @@ def cpu_baseline(torch, sample_tokens):
     rt.swiglu_mlp_fwd_bwd(x, w1, w2, w3, gy)
     dt = time.perf_counter() - t0
     flop = 18 * sample_tokens * DIM * FFN
+    # configs[0], the reference's own CPU-runnable case: one row-wise linear forward, x [4096,2048], W [2048,2048]
+    x1 = torch.randn(4096, 2048, generator=g).to(torch.bfloat16)
+    w1c = (torch.randn(2048, 2048, generator=g) * 0.02).to(torch.bfloat16)
+    reps = []
+    for _ in range(4):
+        t0 = time.perf_counter()
+        rt.linear_forward(x1, w1c)
+        reps.append(time.perf_counter() - t0)
+    c1 = sorted(reps[1:])[1]   # median of three after one warm-up
     return {
         "value": round(flop / dt / 1e12, 4),
         "unit": "TFLOP/s",
@@ -107,6 +121,8 @@ def cpu_baseline(torch, sample_tokens):
         "kind": "port",
         "sample": f"same MLP fwd+bwd on {sample_tokens} of {TOKENS} tokens, one repetition, {dt:.2f} s "
                   f"(PyTorch CPU ops: amax/clamp/div/reciprocal/mul/to(float8_e4m3fn), dequantise, fp32 matmul, bf16)",
+        "config1_linear_forward": {"value": round(2 * 4096 * 2048 * 2048 / c1 / 1e12, 4), "unit": "TFLOP/s",
+                                   "ms": round(c1 * 1e3, 2), "sample": "x [4096,2048] @ W [2048,2048]^T, casts included, median of 3"},
     }
 
 
@@ -147,7 +163,30 @@ def extras(torch, mlp, timed, args):
     return res
 
 
-def run_linear7b(args, torch, dev):
+def more_extras(torch, dev, args):
+    """The other measurements the survey asks for, each freed before the next: one Fp8Linear forward+backward, the
+    config-4 outlier-stress figures (row-wise against tensor-wise scaling) and the Llama-1B-shaped step."""
+    res = {}
+    res["linear7b"] = measure_linear7b(args, torch, dev)
+    torch.cuda.empty_cache()
+    from workloads import outlier_stress_figures
+    fig, tensors = outlier_stress_figures(TOKENS)
+    del tensors
+    torch.cuda.empty_cache()
+    res["config4_outlier_stress"] = dict(fig, what="4096->11008 linear on Student-t(3) activations, 0.1 % of channels x100, "
+                                         "1 % zero rows: SNR of the quantised x and rel-L2 of y against the fp32 product")
+    res["llama1b"] = measure_llama1b(torch, dev, steps=5, warmup=2, fused_too=True)
+    return res
+
+
+def bump_versions(torch, params):
+    """What an optimizer step does to the parameters as far as this library can see: their version counters
+    advance (no device work), so nothing keyed on a weight's version can be reused from the step before."""
+    for p in params:
+        torch.autograd.graph.increment_version(p)
+
+
+def measure_linear7b(args, torch, dev):
     """One Fp8Linear 4096 -> 11008 on 16384 tokens, forward + backward (dgrad + fp8 wgrad), casts included."""
     from lingua_amd import Fp8Linear
     g = torch.Generator().manual_seed(0)
@@ -159,6 +198,7 @@ def run_linear7b(args, torch, dev):
 
     def step():
         lin.weight.grad = x.grad = None
+        bump_versions(torch, [lin.weight])
         lin(x).backward(gy)
 
     for _ in range(args.warmup):
@@ -170,16 +210,23 @@ def run_linear7b(args, torch, dev):
     torch.cuda.synchronize()
     dt = (time.perf_counter() - t0) / args.steps
     flop = 6 * TOKENS * DIM * FFN
+    return {"value": round(flop / dt / 1e12, 2), "unit": "TFLOP/s", "ms_per_step": round(dt * 1e3, 4),
+            "frac_of_fp8_peak": round(flop / dt / 1e12 / PEAK_FP8_TFLOPS, 4), "flop_per_step": flop,
+            "what": "single Fp8Linear 4096->11008 fwd+bwd (dgrad + fp8 wgrad), 16384 tokens, casts included"}
+
+
+def run_linear7b(args, torch, dev):
+    r = measure_linear7b(args, torch, dev)
     print(json.dumps({
-        "metric": "fp8 rowwise linear fwd+bwd TFLOP/s, one 4096->11008 linear", "value": round(flop / dt / 1e12, 2),
-        "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(dt * 1e3, 4),
+        "metric": "fp8 rowwise linear fwd+bwd TFLOP/s, one 4096->11008 linear", "value": r["value"],
+        "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": r["ms_per_step"],
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "fp8_e4m3fn", "data": "synthetic",
-        "config": {"workload": "single Fp8Linear 4096->11008 fwd+bwd, 16384 tokens, casts included", "flop_per_step": flop},
-        "frac_of_fp8_peak": round(flop / dt / 1e12 / PEAK_FP8_TFLOPS, 4),
+        "config": {"workload": r["what"], "flop_per_step": r["flop_per_step"]},
+        "frac_of_fp8_peak": r["frac_of_fp8_peak"],
     }))
 
 
-def run_llama1b(args, torch, dev):
+def measure_llama1b(torch, dev, steps, warmup, fused_too=True):
     """configs[4]: tokens/s of a Llama-1B-shaped forward+backward step, block linears in row-wise fp8."""
     from lingua_amd import convert_linears_to_fp8
     from workloads import Llama, LLAMA_1B, llama_flops_per_token
@@ -193,38 +240,55 @@ def run_llama1b(args, torch, dev):
     labels = torch.randint(0, LLAMA_1B["vocab"], (B, S), generator=g).to(dev)
 
     def timed(m):
+        params = list(m.parameters())
+
         def step():
-            for p in m.parameters():
+            for p in params:
                 p.grad = None
+            bump_versions(torch, params)
             m(tokens, labels).backward()
 
-        for _ in range(args.warmup):
+        for _ in range(warmup):
             step()
         torch.cuda.synchronize()
         t0 = time.perf_counter()
-        for _ in range(args.steps):
+        for _ in range(steps):
             step()
         torch.cuda.synchronize()
-        return (time.perf_counter() - t0) / args.steps
+        return (time.perf_counter() - t0) / steps
 
     dt = timed(model)
     fused_dt = None
-    if not args.no_extras:
+    if fused_too:
         # same weights, gate fused into the casts and norms that hand their output over quantised
         from lingua_amd.norm import fuse_rmsnorm
         from lingua_amd.swiglu import fuse_feed_forward
         fused_dt = timed(fuse_rmsnorm(fuse_feed_forward(model)))
     fpt = llama_flops_per_token(LLAMA_1B["n_layers"], LLAMA_1B["dim"], LLAMA_1B["ffn_dim"], LLAMA_1B["vocab"], S)
     fp8_flop = 25 * 3 * (4 * 2 * B * S * 2048 * 2048 + 3 * 2 * B * S * 2048 * 8192)
+    res = {"value": round(B * S / dt, 1), "unit": "tokens/s", "ms_per_step": round(dt * 1e3, 3), "steps": steps, "warmup": warmup,
+           "model_TFLOP/s": round(fpt * B * S / dt / 1e12, 1), "fp8_linear_TFLOP/s_if_alone": round(fp8_flop / dt / 1e12, 1),
+           "what": "Llama-1B-shaped step fwd+bwd (configs[4]): 25 layers, dim 2048, ffn 8192, vocab 128256, 4 x 4096 tokens; "
+                   "block linears through convert_linears_to_fp8, the rest of the step is the stand-in model's plain PyTorch"}
+    if fused_dt is not None:
+        res["fused_swiglu_and_rmsnorm"] = {"value": round(B * S / fused_dt, 1), "unit": "tokens/s",
+                                           "ms_per_step": round(fused_dt * 1e3, 3)}
+    del model
+    torch.cuda.empty_cache()
+    return res
+
+
+def run_llama1b(args, torch, dev):
+    from workloads import LLAMA_1B
+    r = measure_llama1b(torch, dev, args.steps, args.warmup, fused_too=not args.no_extras)
     print(json.dumps({
-        "metric": "Llama-1B forward+backward tokens/s, block linears fp8 row-wise", "value": round(B * S / dt, 1),
-        "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(dt * 1e3, 3),
+        "metric": "Llama-1B forward+backward tokens/s, block linears fp8 row-wise", "value": r["value"],
+        "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": r["ms_per_step"],
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "fp8_e4m3fn", "data": "synthetic",
-        "config": {"workload": "llama-1B step fwd+bwd (configs[4])", "batch": B, "seq_len": S, **LLAMA_1B},
-        "model_TFLOP/s": round(fpt * B * S / dt / 1e12, 1),
-        "fp8_linear_TFLOP/s_if_alone": round(fp8_flop / dt / 1e12, 1),
-        "extras": None if fused_dt is None else {"fused_swiglu_and_rmsnorm": {
-            "value": round(B * S / fused_dt, 1), "unit": "tokens/s", "ms_per_step": round(fused_dt * 1e3, 3)}},
+        "config": {"workload": "llama-1B step fwd+bwd (configs[4])", "batch": 4, "seq_len": 4096, **LLAMA_1B},
+        "model_TFLOP/s": r["model_TFLOP/s"],
+        "fp8_linear_TFLOP/s_if_alone": r["fp8_linear_TFLOP/s_if_alone"],
+        "extras": {"fused_swiglu_and_rmsnorm": r.get("fused_swiglu_and_rmsnorm")},
     }))
 
 
@@ -318,14 +382,20 @@ def main():
     x = torch.randn(TOKENS, DIM, generator=g).to(torch.bfloat16).to(dev).requires_grad_(True)
     gy = (torch.randn(TOKENS, DIM, generator=g) * 1e-2).to(torch.bfloat16).to(dev)
 
-    def timed(module, records):
+    def make_step(module):
+        params = list(module.parameters())
+
         def step():
-            for p in module.parameters():
+            for p in params:
                 p.grad = None
             x.grad = None
+            bump_versions(torch, params)   # as after an optimizer step: nothing may be reused from the step before
             y = module(x)
             y.backward(gy)
+        return step
 
+    def timed(module, records):
+        step = make_step(module)
         for _ in range(args.warmup):
             step()
         torch.cuda.synchronize()
@@ -338,6 +408,20 @@ def main():
         elapsed = time.perf_counter() - t0
         ops.kernel_timer = None
         return elapsed
+
+    def sustained(module, seconds):
+        """The same step, repeated for at least `seconds` of wall clock: the clock the part settles at under load."""
+        step = make_step(module)
+        n, t0 = 0, time.perf_counter()
+        while True:
+            for _ in range(20):
+                step()
+            n += 20
+            torch.cuda.synchronize()
+            el = time.perf_counter() - t0
+            if el >= seconds:
+                return {"value": round(STEP_FLOP * n / el / 1e12, 2), "unit": "TFLOP/s", "steps": n, "seconds": round(el, 2),
+                        "ms_per_step": round(el / n * 1e3, 4)}
 
     records = None if args.no_kernel_timing else []
     dt = timed(mlp, records)
@@ -390,7 +474,11 @@ def main():
         "kernels": kernels,
     }
     if not args.no_extras:
+        out["sustained"] = sustained(mlp, args.sustained_seconds)
         out["extras"] = extras(torch, mlp, timed, args)
+        del mlp, model, x, gy
+        torch.cuda.empty_cache()
+        out["extras"].update(more_extras(torch, dev, args))
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline(torch, args.cpu_sample_tokens)
     print(json.dumps(out))
