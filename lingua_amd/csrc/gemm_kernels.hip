@@ -923,12 +923,20 @@ template __global__ void gemm_nt_stream_kernel<8, false>(const GemmArgs);
 template __global__ void gemm_nt_stream_kernel<8, true>(const GemmArgs);
 template __global__ void gemm_nt_stream_kernel<4, false>(const GemmArgs);
 template __global__ void gemm_nt_stream_kernel<4, true>(const GemmArgs);
+template __global__ void gemm_nt_stream_kernel<2, false>(const GemmArgs);
+template __global__ void gemm_nt_stream_kernel<2, true>(const GemmArgs);
+template __global__ void gemm_nt_stream_kernel<16, false>(const GemmArgs);
+template __global__ void gemm_nt_stream_kernel<16, true>(const GemmArgs);
 
 static const Algo kAlgos[] = {
     L8_ALGO_LIST(L8_ALGO_ROW)
     /* 11, 12: persistent 256x256 tiles, 4 waves, one panel stream across tiles, C stored from the accumulators */
     {"stream_mt2x2w_4x4t_r5_g8", gemm_nt_stream_kernel<8, false>, 256, 256, 256, 5 * 256 * 128, true, gemm_nt_stream_kernel<8, true>},
     {"stream_mt2x2w_4x4t_r5_g4", gemm_nt_stream_kernel<4, false>, 256, 256, 256, 5 * 256 * 128, true, gemm_nt_stream_kernel<4, true>},
+    /* 13, 14: other shapes of the block of tiles resident on an XCD (2 x 16 and 16 x 2 instead of 4 x 8: 18 panels
+       shared by 32 tiles instead of 12), kept for the traffic comparison */
+    {"stream_mt2x2w_4x4t_r5_g2", gemm_nt_stream_kernel<2, false>, 256, 256, 256, 5 * 256 * 128, true, gemm_nt_stream_kernel<2, true>},
+    {"stream_mt2x2w_4x4t_r5_g16", gemm_nt_stream_kernel<16, false>, 256, 256, 256, 5 * 256 * 128, true, gemm_nt_stream_kernel<16, true>},
 };
 constexpr int kNumAlgos = sizeof(kAlgos) / sizeof(kAlgos[0]);
 
