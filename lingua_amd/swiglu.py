@@ -37,9 +37,17 @@ class Fp8SwiGLUFn(torch.autograd.Function):
         cfg = f8.config
         fp8_wgrad = cfg.fp8_wgrad
         algo = cfg.gemm_algo
-        x_col = torch.empty(x.shape[1], dtype=torch.float32, device=x.device) \
-            if fp8_wgrad and (w1.requires_grad or w3.requires_grad) else None
-        qx, sx, _ = ops.cast_rowwise(x, col_amax=x_col)
+        need_x_col = fp8_wgrad and (w1.requires_grad or w3.requires_grad)
+        # an Fp8RMSNorm in front of this block has filed its output already quantised (with its column amaxes when
+        # it ran in training mode): take that copy instead of quantising the activation a second time
+        hit = f8._fwd_cast.get(x, ("swiglu", w1.data_ptr())) if cfg.share_input_casts else None
+        if hit is not None and (hit[2] is not None or not need_x_col):
+            qx, sx, x_col = hit
+            if not need_x_col:
+                x_col = None
+        else:
+            x_col = torch.empty(x.shape[1], dtype=torch.float32, device=x.device) if need_x_col else None
+            qx, sx, _ = ops.cast_rowwise(x, col_amax=x_col)
         q1, s1, amax_w1 = ops.cast_rowwise(w1)
         q3, s3, amax_w3 = ops.cast_rowwise(w3)
         h1 = ops.gemm_nt(qx, q1, sx, s1, None, algo=algo)

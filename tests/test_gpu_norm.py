@@ -200,3 +200,42 @@ def test_small_llama_with_fused_gate_and_norms_matches_the_drop_in_model():
     for n in ref:
         e_plain, e_fused = rel_l2(plain[n].grad, ref[n].grad), rel_l2(fused[n].grad, ref[n].grad)
         assert e_fused <= 1.25 * e_plain + 1e-3, (n, e_plain, e_fused)
+
+
+def test_fused_feed_forward_takes_the_norm_output_already_quantised():
+    """ffn_norm -> feed_forward with both fused: the norm files its output quantised (with column amaxes in
+    training), and the fused SwiGLU takes that copy instead of casting the activation again -- one row-wise cast
+    fewer per block, identical results (the same kernel arithmetic produced the copy either way)."""
+    from lingua_amd import float8, ops
+    from lingua_amd.norm import Fp8RMSNorm
+    from lingua_amd.swiglu import Fp8FeedForward
+    from workloads import FeedForward
+    torch.manual_seed(4)
+    ff = FeedForward(512, 1024).to(device="cuda", dtype=torch.bfloat16)
+    norm = Fp8RMSNorm(512, 1e-5).to(device="cuda", dtype=torch.bfloat16)
+    fused = Fp8FeedForward(ff.w1, ff.w3, ff.w2)
+    x = seeded_bf16((3, 40, 512), std=1.5, seed=19).cuda()
+    g = seeded_bf16((3, 40, 512), std=0.02, seed=20).cuda()
+
+    def run(share):
+        old = float8.config.share_input_casts
+        float8.config.share_input_casts = share
+        rec = []
+        ops.kernel_timer = rec
+        try:
+            for p in list(ff.parameters()) + [norm.weight]:
+                p.grad = None
+            xi = x.clone().requires_grad_(True)
+            y = fused(norm(xi))
+            n_fwd = sum(1 for r in rec if r[0] == "cast_rowwise")
+            y.backward(g)
+        finally:
+            ops.kernel_timer = None
+            float8.config.share_input_casts = old
+        return [y.detach(), xi.grad] + [p.grad.clone() for p in ff.parameters()], n_fwd
+
+    got, n_shared = run(True)
+    want, n_apart = run(False)
+    assert n_apart == 4 and n_shared == 3          # x + three weights against the three weights only
+    for a, b in zip(got, want):
+        assert torch.equal(a.view(torch.int16), b.view(torch.int16))
