@@ -132,6 +132,23 @@ int l8_gemm_nt(const void *A, const void *B, int64_t M, int64_t N, int64_t K,
                const float *sa, int sa_mode, const float *sb, int sb_mode,
                const void *bias, void *C, int64_t ldc, int algo, void *stream);
 
+/* l8_gemm_nt with a workspace.  Tile configuration 15 (opt-in, never the default) uses it to share the K
+ * range of the last round's tiles out between workgroups when that round would leave part of the GPU idle
+ * (long K, tile count a little above a multiple of the compute units): fp32 partial sums are exchanged
+ * through the workspace and added in a fixed order, so results do not vary from call to call.  Every other
+ * configuration ignores the workspace.  Same replacement as l8_gemm_nt (torch._scaled_mm at
+ * lingua/float8.py:65-77 splits K internally as it sees fit).
+ *   workspace: l8_gemm_workspace() bytes of device memory, 16-byte aligned, ZERO-FILLED ONCE before its
+ *              first use and never written by anyone else afterwards (the library keeps launch numbers in
+ *              it); calls that share a workspace must not overlap in time (one workspace per stream).
+ *              NULL, too small, a bias, or a stream that is being captured: exactly l8_gemm_nt. */
+int l8_gemm_nt_ws(const void *A, const void *B, int64_t M, int64_t N, int64_t K,
+                  int64_t lda, int64_t ldb,
+                  const float *sa, int sa_mode, const float *sb, int sb_mode,
+                  const void *bias, void *C, int64_t ldc, int algo,
+                  void *workspace, int64_t workspace_bytes, void *stream);
+int64_t l8_gemm_workspace(void);
+
 /* SwiGLU gate fused with the row-wise cast of the w2 input.
  * Replaces `F.silu(self.w1(x)) * self.w3(x)` of lingua/transformer.py:469-471 (two bf16
  * elementwise kernels) followed by the cast of that product in Fp8LinearFn.forward

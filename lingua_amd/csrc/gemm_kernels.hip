@@ -47,6 +47,7 @@
 // of the main loop to attribute stalls: 1 = no global loads after the prologue,
 // 2 = no LDS reads / matrix-core work, 3 = no stores of C, 4 = as 2 with every workgroup loading the same tile (all
 // L2 hits).  Results are wrong by construction.
+#include <atomic>
 #include <type_traits>
 
 #include "l8_common.h"
@@ -63,6 +64,11 @@ struct GemmArgs {
   uint16_t *C;
   int tiles_m, tiles_n;
   uint64_t *dbg;  // L8_GEMM_PROF builds only
+  // persistent kernels, optional (null = every tile is computed by one workgroup): workspace for tiles whose
+  // K range is shared out over several workgroups -- one flag and one fp32 tile of partial sums per workgroup
+  uint32_t *sk_flags;
+  float *sk_partials;
+  uint32_t sk_epoch;  // value that marks a flag as set in THIS launch (never 0; flags are never cleared)
 };
 
 typedef __attribute__((address_space(3))) void *lds_ptr_t;
@@ -75,7 +81,13 @@ L8_DEV __amdgpu_buffer_rsrc_t make_rsrc(const void *p, uint32_t bytes) {
 }
 #endif
 
-[[maybe_unused]] constexpr uint32_t kOOB = 0x80000000u;  // voffset that is out of range for every resource below
+[[maybe_unused]] constexpr uint32_t kOOB = 0x80000000u;
+// cache policy of a buffer access that must be coherent over the whole device (sc0 | sc1)
+[[maybe_unused]] constexpr int kCoherent = 1 | 16;
+// Sharing out the K range of the last, partly filled round of tiles: what a partial tile costs its writer and its
+// reader, in K tiles' time (256 KiB leave a compute unit at ~16 bytes per clock), and the least number of K tiles
+// the split must take off the owners of the tail tiles to be used at all.
+[[maybe_unused]] constexpr int kSkWriteCost = 8, kSkFixCost = 4, kSkMinSaved = 16;  // voffset that is out of range for every resource below
 
 #ifndef L8_GEMM_DIAG
 #define L8_GEMM_DIAG 0
@@ -504,7 +516,7 @@ __global__ __launch_bounds__(WM *WN * 64) void gemm_nt_kernel(const GemmArgs p) 
 // so the workgroups resident on an XCD always work on W consecutive tiles of
 // the grouped order and share their panels in that XCD's L2.
 // ---------------------------------------------------------------------------
-template <int GROUP_M, bool HAS_BIAS>
+template <int GROUP_M, bool HAS_BIAS, bool SK = false>
 __global__ __launch_bounds__(256) void gemm_nt_stream_kernel(const GemmArgs p) {
 #if defined(__HIP_DEVICE_COMPILE__)
   constexpr int BM = 256, BN = 256, BK = 128, NW = 4, TM = 4, TN = 4, R = 5;
@@ -526,12 +538,34 @@ __global__ __launch_bounds__(256) void gemm_nt_stream_kernel(const GemmArgs p) {
   const int q = nb >> 3, rem = nb & 7;
   const int first = (xcd < rem) ? xcd * (q + 1) : rem * (q + 1) + (xcd - rem) * q;
   const int cnt = q + (xcd < rem ? 1 : 0);
-  const int n_seg = loc < cnt ? (cnt - loc + W - 1) / W : 0;
-  if (n_seg == 0) return;
-  [[maybe_unused]] uint64_t prof[16] = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
   const int KT = (p.K + BK - 1) / BK;
-  auto tile_of = [&](int seg, int &m0, int &n0) {
-    const int lin = first + loc + seg * W;
+  // SK instantiation -- tail of the XCD's range: the r = cnt % W tiles left after the full rounds would keep r
+  // workgroups busy for a whole K loop and H = W - r idle.  When the idle ones can take enough off the others to
+  // pay for an exchange of partial sums, each tail tile's K range is cut in two at the same place: the last r
+  // workgroups take the first k_split K tiles of one tail tile each, in step with each other like a normal round
+  // (workgroups that are at the same K tile at the same time share their panels in the XCD's L2; a split that
+  // staggers them costs more in panel traffic than it saves), and own the tile; the first H workgroups (helpers)
+  // multiply the remaining K tiles of tail tiles loc, loc + H, ... one after the other, again in step with each
+  // other, and leave fp32 partial sums, which the owners add to their own before they store the tile.  Owners
+  // wait only for workgroups with lower numbers (dispatched earlier), which never wait for anybody.
+  // With m = ceil(r / H) pieces per helper, L K tiles per piece, a partial tile costing a helper about
+  // kSkWriteCost K tiles' time to write and an owner kSkFixCost to add, both finish together when
+  // m * (L + kSkWriteCost) = KT - L + kSkFixCost.
+  const int n_rounds = cnt / W, r_tail = cnt - n_rounds * W, n_help = W - r_tail;
+  const int m_help = (r_tail + n_help - 1) / n_help;
+  const int l_help = (KT + kSkFixCost - m_help * kSkWriteCost) / (m_help + 1);
+  const bool sk = SK && p.sk_partials != nullptr && n_rounds > 0 && r_tail > 0 && l_help >= kSkMinSaved;
+  const int k_split = KT - l_help;
+  const bool helper = loc < n_help;
+  const int n_tail = !sk ? 0 : (helper ? (loc < r_tail ? (r_tail - loc + n_help - 1) / n_help : 0) : 1);  // pieces of this workgroup
+  const int n_seg = sk ? n_rounds : (loc < cnt ? (cnt - loc + W - 1) / W : 0);                              // whole tiles
+  if (n_seg + n_tail == 0) return;
+  [[maybe_unused]] uint64_t prof[16] = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+  if (L8_GEMM_PROF) {
+    prof[0] = __builtin_amdgcn_s_memrealtime();
+    prof[5] = __builtin_readcyclecounter();
+  }
+  auto tile_at = [&](int lin, int &m0, int &n0) {
     const int per_group = GROUP_M * p.tiles_n;
     const int grp = lin / per_group;
     const int first_m = grp * GROUP_M;
@@ -540,6 +574,16 @@ __global__ __launch_bounds__(256) void gemm_nt_stream_kernel(const GemmArgs p) {
     m0 = (first_m + in_grp % gsz) * BM;
     n0 = (in_grp / gsz) * BN;
   };
+  auto tile_of = [&](int seg, int &m0, int &n0) { tile_at(first + loc + seg * W, m0, n0); };
+  // piece pc of the tail (highest tile first): tile origin, K-tile range [kb, ke); returns the tail tile's number
+  // piece pc of this workgroup's tail: the tail tile's number (tile origin in m0, n0); every piece of a workgroup
+  // covers the same K tiles [piece_kb, piece_ke)
+  const int piece_kb = helper ? k_split : 0, piece_ke = helper ? KT : k_split;
+  auto piece_of = [&](int pc, int &m0, int &n0) -> int {
+    const int tt = helper ? loc + pc * n_help : loc - n_help;
+    tile_at(first + n_rounds * W + tt, m0, n0);
+    return tt;
+  };
 
   // ---- global -> LDS load plan ----
   // lane l of a wave load fills LDS row l/8, position l%8 of an 8-row group; position p of LDS row r holds
@@ -547,20 +591,47 @@ __global__ __launch_bounds__(256) void gemm_nt_stream_kernel(const GemmArgs p) {
   // g = wave * NL + i.  For the A panel LDS row = tile row.  For the B panel LDS row r = span*128 + tn*32 + j
   // holds tile row span*128 + 4*j + tn: within a group (8 consecutive j) the rows are 4 apart, and the
   // group's first row is span*128 + 4*(8*(g%4)) + (g%16)/4.
-  const int lrow = lane >> 3, lpos = lane & 7;
-  const uint32_t a_voff[2] = {(uint32_t)(lrow * (int)p.lda + (lpos ^ lrow) * 16), (uint32_t)(lrow * (int)p.lda + (lpos ^ lrow ^ 1) * 16)};
-  const uint32_t b_voff[2] = {(uint32_t)(lrow * 4 * (int)p.ldb + (lpos ^ lrow) * 16), (uint32_t)(lrow * 4 * (int)p.ldb + (lpos ^ lrow ^ 1) * 16)};
-  const int chunk_even = (lpos ^ lrow) * 16, chunk_odd = (lpos ^ lrow ^ 1) * 16;
+  // The per-lane constants of the K loop are formed afresh, from an opaque copy of the lane number, in front of
+  // every tile's K loop: values that lived across the conversion of the C tile (the point of highest register
+  // pressure) were the ones the allocator chose to spill, and it reloaded them inside the K loop.
+  uint32_t a_voff[2], b_voff[2], foff[2][2];
+  int chunk_even, chunk_odd;
+  auto lane_consts = [&]() {
+    int l = lane;
+    asm volatile("" : "+v"(l));
+    const int lrow = l >> 3, lpos = l & 7;
+    chunk_even = (lpos ^ lrow) * 16;
+    chunk_odd = (lpos ^ lrow ^ 1) * 16;
+    a_voff[0] = (uint32_t)(lrow * (int)p.lda + chunk_even);
+    a_voff[1] = (uint32_t)(lrow * (int)p.lda + chunk_odd);
+    b_voff[0] = (uint32_t)(lrow * 4 * (int)p.ldb + chunk_even);
+    b_voff[1] = (uint32_t)(lrow * 4 * (int)p.ldb + chunk_odd);
+    const int l31 = l & 31, h = l >> 5;
+    const int fr = (l31 & 7) ^ ((l31 >> 3) & 1);
+#pragma unroll
+    for (int s = 0; s < 2; ++s)
+#pragma unroll
+      for (int j = 0; j < 2; ++j) foff[s][j] = l31 * BK + (((s * 4 + h * 2 + j) ^ fr) * 16);
+  };
+  lane_consts();
   const uint32_t lds0 = (uint32_t)(uintptr_t)(lds_ptr_t)smem;
   auto wrap = [](int slot) { return slot >= R ? slot - R : slot; };
 
   // loader cursor: the K tile whose panels are requested next (two K tiles ahead of the one being multiplied)
   int ld_seg = 0, ld_kt = 0;
+  [[maybe_unused]] int ld_ke = KT;  // SK: the loader's piece ends here
   __amdgpu_buffer_rsrc_t ld_rsA, ld_rsB;
   auto ld_open = [&](int seg) {
-    if (seg < n_seg) {
+    if (seg < n_seg + n_tail) {
       int m0, n0;
-      tile_of(seg, m0, n0);
+      if (!SK || seg < n_seg) {
+        tile_of(seg, m0, n0);
+        if (SK) ld_ke = KT;
+      } else {
+        piece_of(seg - n_seg, m0, n0);
+        ld_kt = piece_kb;
+        ld_ke = piece_ke;
+      }
       const int64_t a_left = (int64_t)(p.M - m0 - 1) * p.lda + p.K;
       const int64_t b_left = (int64_t)(p.N - n0 - 1) * p.ldb + p.K;
       ld_rsA = make_rsrc(p.A + (int64_t)m0 * p.lda, a_left < 0x7fffffff ? (uint32_t)a_left : 0x7fffffffu);
@@ -568,10 +639,11 @@ __global__ __launch_bounds__(256) void gemm_nt_stream_kernel(const GemmArgs p) {
     } else {  // past the last tile: every load is out of range and fills its LDS bytes with zeros
       ld_rsA = make_rsrc(p.A, 0);
       ld_rsB = make_rsrc(p.B, 0);
+      if (SK) ld_ke = 0x7fffffff;
     }
   };
   auto ld_advance = [&]() {
-    if (++ld_kt == KT) {
+    if (++ld_kt == (SK ? ld_ke : KT)) {
       ld_kt = 0;
       ld_open(++ld_seg);
     }
@@ -593,12 +665,6 @@ __global__ __launch_bounds__(256) void gemm_nt_stream_kernel(const GemmArgs p) {
 
   // ---- LDS -> register fragment plan (as in the kernel above) ----
   const int l31 = lane & 31, h = lane >> 5;
-  const int fr = (l31 & 7) ^ ((l31 >> 3) & 1);
-  uint32_t foff[2][2];
-#pragma unroll
-  for (int s = 0; s < 2; ++s)
-#pragma unroll
-    for (int j = 0; j < 2; ++j) foff[s][j] = l31 * BK + (((s * 4 + h * 2 + j) ^ fr) * 16);
   const int a_base = wm * (TM * 32 * BK);
   const int b_base = wn * (TN * 32 * BK);
   typedef const __attribute__((address_space(3))) v4i *lds_v4i_ptr;
@@ -633,6 +699,14 @@ __global__ __launch_bounds__(256) void gemm_nt_stream_kernel(const GemmArgs p) {
     acc[tm][tn] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(af[tm], bf[tn], acc[tm][tn], 0, 0, 0, 0, 0, 0);
   };
 
+  // One accumulator element, fetched where it is used.  Written as assembly with an accumulator-register operand:
+  // given plain reads, the register allocator moves the whole accumulator set into ordinary vector registers in
+  // front of the conversion of the C tile and pays for it with spills inside the K loop.
+  auto acc_read = [&](int tm, int tn, int i) -> float {
+    float x;
+    asm volatile("v_accvgpr_read_b32 %0, %1" : "=v"(x) : "a"(acc[tm][tn][i]));
+    return x;
+  };
   // ---- C tile straight from the accumulators ----
   // acc[tm][tn][4*qd + e] of lane (l31, h) is C[m][n] with m = wm*128 + tm*32 + 8*qd + 4*h + e and
   // n = wn*128 + 4*l31 + tn (tile coordinates).  The host launches this kernel only when every lane pair's
@@ -645,9 +719,7 @@ __global__ __launch_bounds__(256) void gemm_nt_stream_kernel(const GemmArgs p) {
   int seg_sa[2] = {0, 0};
   v4i seg_sb = {0, 0, 0, 0};
   [[maybe_unused]] v2i seg_bias = {0, 0};
-  auto load_scales = [&](int seg) {
-    int m0, n0;
-    tile_of(seg, m0, n0);
+  auto load_scales = [&](int m0, int n0) {
     const int64_t sa_left = (int64_t)(p.M - m0) * 4, sb_left = (int64_t)(p.N - n0) * 4;
     if (p.sa_row) {
       const __amdgpu_buffer_rsrc_t rsSa = make_rsrc(p.sa + m0, sa_left < 0x7fffffff ? (uint32_t)sa_left : 0x7fffffffu);
@@ -670,9 +742,17 @@ __global__ __launch_bounds__(256) void gemm_nt_stream_kernel(const GemmArgs p) {
   };
   // (A compute unit drains its stores at about 16 bytes per clock: the 128 KiB of a C tile keep it busy for some
   // 8000 cycles, of which the conversion below hides about half.)
-  auto store_tile = [&](int seg) {
-    int m0, n0;
-    tile_of(seg, m0, n0);
+  // PARTS (a tile whose last K tiles were multiplied by another workgroup): rs_p is the partial sum over those K
+  // tiles, added to the workgroup's own.
+  // Byte offset of piece i (of 64) of this wave in a slot.  The slots are 256 KiB apart and the workgroups of a
+  // launch write theirs in step: the pieces are rotated by the slot number so that stores issued at the same time
+  // do not all fall on the same memory channels.
+  [[maybe_unused]] auto piece_off = [&](int slot, int i) { return (wave * (TM * TN * 4) + ((i + slot * 5) & (TM * TN * 4 - 1))) * 1024; };
+  [[maybe_unused]] __amdgpu_buffer_rsrc_t rs_p;
+  [[maybe_unused]] int p_slot = 0;
+  constexpr int P_AHEAD = 3;  // groups / pieces of the partial sum requested ahead of their use (their latency is long)
+  auto store_tile = [&](int m0, int n0, auto parts_tag) {
+    constexpr bool PARTS = decltype(parts_tag)::value;
     // Opaque copies: everything below would otherwise be hoisted out of the K loop as loop-invariant (row
     // offsets in scalar registers, per-lane addresses in vector registers) and held across it.
     int ldc2 = (int)p.ldc * 2;
@@ -697,6 +777,7 @@ __global__ __launch_bounds__(256) void gemm_nt_stream_kernel(const GemmArgs p) {
     // precomputed into 64 registers and spilled) and are waited for by hand: LDS operations return in order, so
     // "at most 4 outstanding" means that everything but the group requested last has arrived.
     const int sa_addr = 16 * h;  // byte address of lane 4*h
+    const int sa_regs[2] = {seg_sa[0], seg_sa[1]};
     float sa_grp[2][4];
     auto request_row_scales = [&](int g, float (&dst)[4]) {  // g = tm * 4 + qd
       const int tm = g >> 2, qd = g & 3;
@@ -704,9 +785,24 @@ __global__ __launch_bounds__(256) void gemm_nt_stream_kernel(const GemmArgs p) {
       for (int e = 0; e < 4; ++e)
         asm volatile("ds_bpermute_b32 %0, %1, %2 offset:%3"
                      : "=v"(dst[e])
-                     : "v"(sa_addr), "v"(seg_sa[tm >> 1]), "n"(4 * ((tm & 1) * 32 + 8 * qd + e)));
+                     : "v"(sa_addr), "v"(sa_regs[tm >> 1]), "n"(4 * ((tm & 1) * 32 + 8 * qd + e)));
     };
     request_row_scales(0, sa_grp[0]);
+    // partial sums of the group (tm, qd): one 16-byte piece per lane and accumulator, laid out as write_partial
+    // stores them; requested P_AHEAD groups ahead
+    [[maybe_unused]] v4f pbuf[P_AHEAD + 1][TN];
+    [[maybe_unused]] const int p_voff = lane * 16;
+    [[maybe_unused]] auto request_parts = [&](int g, v4f (&dst)[TN]) {
+      const int tm = g >> 2, qd = g & 3;
+#pragma unroll
+      for (int tn = 0; tn < TN; ++tn)
+        dst[tn] = __builtin_bit_cast(v4f, __builtin_amdgcn_raw_buffer_load_b128(
+                                              rs_p, p_voff, piece_off(p_slot, (tm * TN + tn) * 4 + qd), kCoherent));
+    };
+    if constexpr (PARTS) {
+#pragma unroll
+      for (int g = 0; g < P_AHEAD; ++g) request_parts(g, pbuf[g]);
+    }
     [[maybe_unused]] uint64_t tq0 = 0, tq1 = 0, tq2 = 0;
     if (L8_GEMM_PROF) {
       tq0 = __builtin_readcyclecounter();
@@ -733,6 +829,9 @@ __global__ __launch_bounds__(256) void gemm_nt_stream_kernel(const GemmArgs p) {
         const int row = wm * 128 + tm * 32 + 8 * qd;  // + 4*h + e
         const int g = tm * 4 + qd;
         float(&sa_cur)[4] = sa_grp[g & 1];
+        if constexpr (PARTS) {
+          if (g + P_AHEAD < TM * 4) request_parts(g + P_AHEAD, pbuf[(g + P_AHEAD) % (P_AHEAD + 1)]);
+        }
         if (g + 1 < TM * 4) {
           request_row_scales(g + 1, sa_grp[(g + 1) & 1]);
           asm volatile("s_waitcnt lgkmcnt(4)" : "+v"(sa_cur[0]), "+v"(sa_cur[1]), "+v"(sa_cur[2]), "+v"(sa_cur[3]));
@@ -748,7 +847,9 @@ __global__ __launch_bounds__(256) void gemm_nt_stream_kernel(const GemmArgs p) {
             float v[4];
 #pragma unroll
             for (int tn = 0; tn < TN; ++tn) {
-              v[tn] = acc[tm][tn][4 * qd + e2 + r] * sa * sbv[tn];
+              float a = acc_read(tm, tn, 4 * qd + e2 + r);
+              if constexpr (PARTS) a = a + pbuf[g % (P_AHEAD + 1)][tn][e2 + r];  // ascending K
+              v[tn] = a * sa * sbv[tn];
               if constexpr (HAS_BIAS) v[tn] += bv[tn];
             }
             typedef __bf16 bf2 __attribute__((ext_vector_type(2)));
@@ -762,6 +863,9 @@ __global__ __launch_bounds__(256) void gemm_nt_stream_kernel(const GemmArgs p) {
           const int got1 = __builtin_amdgcn_update_dpp(0, give1, 0xB1, 0xF, 0xF, true);
           const v4i out = par ? v4i{got0, got1, o[1][0], o[1][1]} : v4i{o[0][0], o[0][1], got0, got1};
           __builtin_amdgcn_raw_buffer_store_b128(out, rsC, c_voff, (row + e2) * ldc2, 2 /* streaming */);
+          // one row pair at a time: left free, the scheduler reads a hundred accumulator registers ahead and the
+          // register pressure of this conversion makes the allocator spill values the K loop uses in every trip
+          __builtin_amdgcn_sched_barrier(0);
         }
       }
     }
@@ -775,6 +879,55 @@ __global__ __launch_bounds__(256) void gemm_nt_stream_kernel(const GemmArgs p) {
       for (int tn = 0; tn < TN; ++tn)
 #pragma unroll
         for (int v = 0; v < 16; ++v) acc[tm][tn][v] = 0.0f;
+  };
+
+  // ---- SK: exchange of partial sums for tiles whose K range is shared out ----
+  // Tail tile tt of XCD x has flag sk_flags[tt * 8 + x] and the fp32 tile sk_partials[(tt * 8 + x) * 65536 ...],
+  // laid out the way the accumulators are held (one 16-byte piece per lane, wave, accumulator and quad: whole KiB per wave store).
+  // Partial sums and flags are written and read with device-coherent accesses (they bypass the caches that are
+  // not shared by all compute units), so no cache needs flushing or invalidating: a wave waits until its own
+  // stores are acknowledged, the workgroup meets at a barrier, and one lane then raises the flag.
+  [[maybe_unused]] auto partial_rsrc = [&](int slot) {
+    return make_rsrc(p.sk_partials + (int64_t)slot * (BM * BN), BM * BN * 4);
+  };
+  [[maybe_unused]] auto write_partial = [&](int slot) {
+    constexpr int N_PIECES = TM * TN * 4;
+    const __amdgpu_buffer_rsrc_t rs = partial_rsrc(slot);
+    const int voff = lane * 16;
+#pragma unroll
+    for (int tm = 0; tm < TM; ++tm)
+#pragma unroll
+      for (int tn = 0; tn < TN; ++tn) {
+#pragma unroll
+        for (int qd = 0; qd < 4; ++qd) {
+          const v4f v = {acc_read(tm, tn, 4 * qd), acc_read(tm, tn, 4 * qd + 1), acc_read(tm, tn, 4 * qd + 2), acc_read(tm, tn, 4 * qd + 3)};
+          __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(v4i, v), rs, voff, piece_off(slot, (tm * TN + tn) * 4 + qd), kCoherent);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+      }
+#pragma unroll
+    for (int tm = 0; tm < TM; ++tm)
+#pragma unroll
+      for (int tn = 0; tn < TN; ++tn)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) acc[tm][tn][v] = 0.0f;
+    L8_WAIT_VM_LGKM0(0);  // this wave's part of the tile has reached the point of coherence
+    asm volatile("" ::: "memory");
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
+    if (threadIdx.x == 0) __hip_atomic_store(p.sk_flags + slot, p.sk_epoch, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  };
+  // Wait until the partial sums in `slot` have been published in this launch.  Their maker has a lower number
+  // than the caller (dispatched earlier) and never waits for anybody.  The wait is bounded all the same: a flag
+  // that never comes poisons the tile with a NaN instead of hanging the GPU.
+  [[maybe_unused]] auto wait_partial = [&](int slot) -> bool {
+#pragma unroll 1
+    for (int spin = 0; spin < (1 << 18); ++spin) {
+      const uint32_t f = __hip_atomic_load(p.sk_flags + slot, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      if ((uint32_t)__builtin_amdgcn_readfirstlane((int)f) == p.sk_epoch) return true;
+      __builtin_amdgcn_s_sleep(32);
+    }
+    return false;
   };
 
   if (L8_GEMM_DIAG == 5 || L8_GEMM_DIAG == 6) {  // experiments: XCD x starts x/8 of a tile's duration late (5); workgroup loc of an XCD starts loc/256 of it late (6)
@@ -849,7 +1002,10 @@ __global__ __launch_bounds__(256) void gemm_nt_stream_kernel(const GemmArgs p) {
       if (seg == 0) prof[1] = __builtin_amdgcn_s_memrealtime();
       t_loop = __builtin_readcyclecounter();
     }
-    load_scales(seg);
+    int m0, n0;
+    tile_of(seg, m0, n0);
+    if (seg > 0) lane_consts();
+    load_scales(m0, n0);
     int kt = 0;
     if (seg > 0) {
       // The first barrier after the N_STORES stores of a C tile: they are younger than the panels waited for
@@ -865,8 +1021,48 @@ __global__ __launch_bounds__(256) void gemm_nt_stream_kernel(const GemmArgs p) {
       prof[3] += t - t_loop;
       t_loop = t;
     }
-    store_tile(seg);
+    store_tile(m0, n0, std::false_type{});
     if (L8_GEMM_PROF) prof[4] += __builtin_readcyclecounter() - t_loop;
+  }
+  if (L8_GEMM_PROF) prof[11] = __builtin_amdgcn_s_memrealtime();
+  if constexpr (SK) {
+    // ---- the workgroup's share of the tail ----
+    bool after_store = true;  // the segment before ended with the N_STORES stores of a C tile (n_seg > 0 here)
+#pragma unroll 1
+    for (int pc = 0; pc < n_tail; ++pc) {
+      int m0, n0;
+      const int tt = piece_of(pc, m0, n0);
+      const bool owns = !helper;  // the tile's first K tiles: this workgroup adds the helper's sums and stores the tile
+      const int slot = tt * 8 + xcd;
+      lane_consts();
+      if (owns) load_scales(m0, n0);
+      [[maybe_unused]] uint64_t t_a = 0, t_b = 0;
+      if (L8_GEMM_PROF) t_a = __builtin_readcyclecounter();
+      if (after_store) trip(integral_constant<int, N_STORES + PEND>{});
+      else trip(integral_constant<int, PEND>{});  // write_partial waited for everything in flight
+#pragma unroll 1
+      for (int kt = piece_kb + 1; kt < piece_ke; ++kt) trip(integral_constant<int, PEND>{});
+      if (L8_GEMM_PROF) {
+        t_b = __builtin_readcyclecounter();
+        prof[12] += t_b - t_a;
+      }
+      if (!owns) {
+        write_partial(slot);
+        after_store = false;
+        if (L8_GEMM_PROF) prof[13] += __builtin_readcyclecounter() - t_b;
+      } else {
+        if (!wait_partial(slot)) seg_sa[0] = seg_sa[1] = 0x7fc00000;  // every row scale a NaN
+        if (L8_GEMM_PROF) {
+          t_a = __builtin_readcyclecounter();
+          prof[14] += t_a - t_b;
+        }
+        rs_p = partial_rsrc(slot);
+        p_slot = slot;
+        store_tile(m0, n0, std::true_type{});
+        after_store = true;
+        if (L8_GEMM_PROF) prof[15] += __builtin_readcyclecounter() - t_a;
+      }
+    }
   }
   // the tail requests (out of range, zero filling) must have landed before the workgroup's LDS is released
   L8_WAIT_VM_LGKM0(0);
@@ -895,6 +1091,7 @@ struct Algo {
   int bm, bn, threads, lds;
   bool persistent;   // one workgroup per compute unit walks a list of tiles
   gemm_fn fn_bias;   // persistent kernels: the instantiation that adds a bias (the plain kernels branch inside)
+  gemm_fn fn_sk;     // persistent kernels: the instantiation that can share a tile's K range out (bias-free), or null
 };
 
 // X(WM, WN, TM, TN, R, GROUP_M, PF) -- 1-based position in this list is the `algo` number
@@ -917,12 +1114,13 @@ L8_ALGO_LIST(L8_INSTANTIATE)
 #define L8_MAX2(a, b) ((a) > (b) ? (a) : (b))
 #define L8_ALGO_ROW(WM, WN, TM, TN, R, GM, PF)                                                                \
   {"mt" #WM "x" #WN "w_" #TM "x" #TN "t_r" #R "_g" #GM "_pf" #PF, gemm_nt_kernel<WM, WN, TM, TN, R, GM, PF>, \
-   WM * TM * 32, WN * TN * 32, WM * WN * 64, R * L8_MAX2(WM * TM * 32, WN * TN * 32) * 128, false, nullptr},
+   WM * TM * 32, WN * TN * 32, WM * WN * 64, R * L8_MAX2(WM * TM * 32, WN * TN * 32) * 128, false, nullptr, nullptr},
 
 template __global__ void gemm_nt_stream_kernel<8, false>(const GemmArgs);
 template __global__ void gemm_nt_stream_kernel<8, true>(const GemmArgs);
 template __global__ void gemm_nt_stream_kernel<4, false>(const GemmArgs);
 template __global__ void gemm_nt_stream_kernel<4, true>(const GemmArgs);
+template __global__ void gemm_nt_stream_kernel<4, false, true>(const GemmArgs);
 template __global__ void gemm_nt_stream_kernel<2, false>(const GemmArgs);
 template __global__ void gemm_nt_stream_kernel<2, true>(const GemmArgs);
 template __global__ void gemm_nt_stream_kernel<16, false>(const GemmArgs);
@@ -931,12 +1129,18 @@ template __global__ void gemm_nt_stream_kernel<16, true>(const GemmArgs);
 static const Algo kAlgos[] = {
     L8_ALGO_LIST(L8_ALGO_ROW)
     /* 11, 12: persistent 256x256 tiles, 4 waves, one panel stream across tiles, C stored from the accumulators */
-    {"stream_mt2x2w_4x4t_r5_g8", gemm_nt_stream_kernel<8, false>, 256, 256, 256, 5 * 256 * 128, true, gemm_nt_stream_kernel<8, true>},
-    {"stream_mt2x2w_4x4t_r5_g4", gemm_nt_stream_kernel<4, false>, 256, 256, 256, 5 * 256 * 128, true, gemm_nt_stream_kernel<4, true>},
+    {"stream_mt2x2w_4x4t_r5_g8", gemm_nt_stream_kernel<8, false>, 256, 256, 256, 5 * 256 * 128, true, gemm_nt_stream_kernel<8, true>, nullptr},
+    {"stream_mt2x2w_4x4t_r5_g4", gemm_nt_stream_kernel<4, false>, 256, 256, 256, 5 * 256 * 128, true, gemm_nt_stream_kernel<4, true>, nullptr},
     /* 13, 14: other shapes of the block of tiles resident on an XCD (2 x 16 and 16 x 2 instead of 4 x 8: 18 panels
        shared by 32 tiles instead of 12), kept for the traffic comparison */
-    {"stream_mt2x2w_4x4t_r5_g2", gemm_nt_stream_kernel<2, false>, 256, 256, 256, 5 * 256 * 128, true, gemm_nt_stream_kernel<2, true>},
-    {"stream_mt2x2w_4x4t_r5_g16", gemm_nt_stream_kernel<16, false>, 256, 256, 256, 5 * 256 * 128, true, gemm_nt_stream_kernel<16, true>},
+    {"stream_mt2x2w_4x4t_r5_g2", gemm_nt_stream_kernel<2, false>, 256, 256, 256, 5 * 256 * 128, true, gemm_nt_stream_kernel<2, true>, nullptr},
+    {"stream_mt2x2w_4x4t_r5_g16", gemm_nt_stream_kernel<16, false>, 256, 256, 256, 5 * 256 * 128, true, gemm_nt_stream_kernel<16, true>, nullptr},
+    /* 15: algo 12 that may share the K range of the last round's tiles out between workgroups (l8_gemm_nt_ws with
+       a workspace; without one it is algo 12).  Measured neutral on the shapes it applies to: the part is
+       power-limited, and the compute units that the plain split leaves idle in the last round let the busy ones
+       clock higher, which recovers most of what the idle ones lose. */
+    {"stream_mt2x2w_4x4t_r5_g4_sk", gemm_nt_stream_kernel<4, false>, 256, 256, 256, 5 * 256 * 128, true, gemm_nt_stream_kernel<4, true>,
+     gemm_nt_stream_kernel<4, false, true>},
 };
 constexpr int kNumAlgos = sizeof(kAlgos) / sizeof(kAlgos[0]);
 
@@ -964,9 +1168,27 @@ static int pick_algo(int64_t M, int64_t N, int64_t K) {
   return 2;
 }
 
-extern "C" int l8_gemm_nt(const void *A, const void *B, int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldb,
-                          const float *sa, int sa_mode, const float *sb, int sb_mode, const void *bias, void *C,
-                          int64_t ldc, int algo, void *stream) {
+// flags (one 4-byte word per workgroup, first 4 KiB) + one fp32 256x256 tile per workgroup of a persistent launch
+constexpr int64_t kSkMaxGrid = 1024, kSkFlagBytes = kSkMaxGrid * 4, kSkTileBytes = 256 * 256 * 4;
+static std::atomic<uint32_t> g_sk_epoch{0};
+
+extern "C" int64_t l8_gemm_workspace(void) {
+  const int64_t cus8 = (num_cus() / 8) * 8;
+  return kSkFlagBytes + (cus8 < 8 ? 8 : cus8) * kSkTileBytes;
+}
+
+// Does sharing out the K range of the last round's tiles pay for an XCD with `cnt` tiles, W workgroups and KT K
+// tiles per tile?  (Same test as in the kernel.)
+static bool sk_pays(int64_t cnt, int64_t W, int64_t KT) {
+  const int64_t n_rounds = cnt / W, r = cnt % W, n_help = W - r;
+  const int64_t m_help = (r + n_help - 1) / n_help;
+  const int64_t l_help = (KT + kSkFixCost - m_help * kSkWriteCost) / (m_help + 1);
+  return n_rounds > 0 && r > 0 && l_help >= kSkMinSaved;
+}
+
+static int gemm_nt_impl(const void *A, const void *B, int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldb,
+                        const float *sa, int sa_mode, const float *sb, int sb_mode, const void *bias, void *C,
+                        int64_t ldc, int algo, void *workspace, int64_t workspace_bytes, void *stream) {
   L8_REQUIRE(M >= 0 && N >= 0 && K >= 0, "l8_gemm_nt: negative shape");
   if (M == 0 || N == 0) return L8_OK;
   L8_REQUIRE(A && B && C && sa && sb, "l8_gemm_nt: null pointer");
@@ -1007,6 +1229,9 @@ extern "C" int l8_gemm_nt(const void *A, const void *B, int64_t M, int64_t N, in
   p.sa_row = sa_mode == L8_SCALE_ROW;
   p.sb_row = sb_mode == L8_SCALE_ROW;
   p.bias = (const uint16_t *)bias;
+  p.sk_flags = nullptr;
+  p.sk_partials = nullptr;
+  p.sk_epoch = 0;
   p.dbg = nullptr;
   if (L8_GEMM_PROF && al.persistent) {
     p.dbg = (uint64_t *)bias;
@@ -1022,6 +1247,7 @@ extern "C" int l8_gemm_nt(const void *A, const void *B, int64_t M, int64_t N, in
   if (slot < 0 || !attr_done[slot][algo - 1]) {
     L8_HIP(hipFuncSetAttribute((const void *)al.fn, hipFuncAttributeMaxDynamicSharedMemorySize, al.lds));
     if (al.fn_bias) L8_HIP(hipFuncSetAttribute((const void *)al.fn_bias, hipFuncAttributeMaxDynamicSharedMemorySize, al.lds));
+    if (al.fn_sk) L8_HIP(hipFuncSetAttribute((const void *)al.fn_sk, hipFuncAttributeMaxDynamicSharedMemorySize, al.lds));
     if (slot >= 0) attr_done[slot][algo - 1] = true;
   }
   int64_t grid = nblocks;
@@ -1032,8 +1258,45 @@ extern "C" int l8_gemm_nt(const void *A, const void *B, int64_t M, int64_t N, in
     grid = want < cus8 ? want : cus8;
     if (grid < 8) grid = 8;
   }
-  const gemm_fn fn = (al.fn_bias && p.bias) ? al.fn_bias : al.fn;
+  gemm_fn fn = (al.fn_bias && p.bias) ? al.fn_bias : al.fn;
+  if (al.fn_sk && !p.bias && workspace != nullptr && grid <= kSkMaxGrid && workspace_bytes >= kSkFlagBytes + grid * kSkTileBytes) {
+    // the kernel decides per XCD (their tile counts differ by at most one) with the same test
+    const int64_t W = grid / 8, KT = (K + 127) / 128, q = nblocks / 8;
+    bool use = sk_pays(q, W, KT) || (nblocks % 8 != 0 && sk_pays(q + 1, W, KT));
+    if (use) {
+      // Not inside a stream capture: the launch number is a kernel argument, and a replayed launch would find
+      // the flags of the replay before already at its number.
+      hipStreamCaptureStatus cs = hipStreamCaptureStatusNone;
+      if (hipStreamIsCapturing((hipStream_t)stream, &cs) != hipSuccess) {
+        (void)hipGetLastError();
+        use = false;
+      } else if (cs != hipStreamCaptureStatusNone) {
+        use = false;
+      }
+    }
+    if (use) {
+      fn = al.fn_sk;
+      p.sk_flags = (uint32_t *)workspace;
+      p.sk_partials = (float *)((uint8_t *)workspace + kSkFlagBytes);
+      uint32_t e = ++g_sk_epoch;
+      if (e == 0) e = ++g_sk_epoch;  // 0 is what an untouched flag holds
+      p.sk_epoch = e;
+    }
+  }
   hipLaunchKernelGGL(fn, dim3((unsigned)grid), dim3(al.threads), al.lds, (hipStream_t)stream, p);
   L8_HIP(hipGetLastError());
   return L8_OK;
+}
+
+extern "C" int l8_gemm_nt(const void *A, const void *B, int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldb,
+                          const float *sa, int sa_mode, const float *sb, int sb_mode, const void *bias, void *C,
+                          int64_t ldc, int algo, void *stream) {
+  return gemm_nt_impl(A, B, M, N, K, lda, ldb, sa, sa_mode, sb, sb_mode, bias, C, ldc, algo, nullptr, 0, stream);
+}
+
+extern "C" int l8_gemm_nt_ws(const void *A, const void *B, int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldb,
+                             const float *sa, int sa_mode, const float *sb, int sb_mode, const void *bias, void *C,
+                             int64_t ldc, int algo, void *workspace, int64_t workspace_bytes, void *stream) {
+  L8_REQUIRE(workspace == nullptr || ((uintptr_t)workspace % 16) == 0, "l8_gemm_nt_ws: workspace must be 16-byte aligned");
+  return gemm_nt_impl(A, B, M, N, K, lda, ldb, sa, sa_mode, sb, sb_mode, bias, C, ldc, algo, workspace, workspace_bytes, stream);
 }

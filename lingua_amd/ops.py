@@ -204,6 +204,25 @@ def cast_colwise_transposed(x: torch.Tensor, col_amax_f32: torch.Tensor, pad_to:
     return q, scale
 
 
+# Tile configuration that may share the K range of the last round's tiles out (opt-in: measured neutral), and its
+# workspace: one per (device, stream), zero-filled when it is made, then owned by the library.
+GEMM_ALGO_SHARED_K = 15
+_gemm_workspaces = {}
+
+
+def _gemm_workspace(device: torch.device, stream_ptr, algo: int):
+    if algo != GEMM_ALGO_SHARED_K:
+        return None, 0
+    key = (device.index, stream_ptr)
+    ws = _gemm_workspaces.get(key)
+    if ws is None:
+        if torch.cuda.is_current_stream_capturing():
+            return None, 0  # no allocation (and no fill) inside a capture; the library takes its plain path
+        ws = torch.zeros(_lib.load().l8_gemm_workspace(), dtype=torch.uint8, device=device)
+        _gemm_workspaces[key] = ws
+    return ws.data_ptr(), ws.numel()
+
+
 def gemm_nt(qa: torch.Tensor, qb: torch.Tensor, sa: torch.Tensor, sb: torch.Tensor,
             bias: Optional[torch.Tensor] = None, algo: int = 0, out: Optional[torch.Tensor] = None) -> torch.Tensor:
     """bf16( (qa @ qb^T) * sa * sb^T + bias ).  qa [M,K], qb [N,K] fp8; sa [M,1]|[1,1], sb [N,1]|[1,1] fp32."""
@@ -228,11 +247,12 @@ def gemm_nt(qa: torch.Tensor, qb: torch.Tensor, sa: torch.Tensor, sb: torch.Tens
         out = torch.empty((M, N), dtype=torch.bfloat16, device=qa.device)
     elif out.dtype != torch.bfloat16 or out.shape != (M, N) or out.stride(1) != 1:
         raise RuntimeError("gemm_nt: out must be bf16 [M,N] with unit column stride")
+    ws_ptr, ws_bytes = _gemm_workspace(qa.device, st, algo)
     with _timed("gemm_nt", 2 * M * N * K, qa.device):
-        code = _lib.load().l8_gemm_nt(qa.data_ptr(), qb.data_ptr(), M, N, K, _ld(qa), _ld(qb), sa.data_ptr(), sa_mode,
-                                      sb.data_ptr(), sb_mode, bias.data_ptr() if bias is not None else None,
-                                      out.data_ptr(), _ld(out) if M > 1 else max(N, 1), algo, st)
-    _lib.check(code, "l8_gemm_nt")
+        code = _lib.load().l8_gemm_nt_ws(qa.data_ptr(), qb.data_ptr(), M, N, K, _ld(qa), _ld(qb), sa.data_ptr(), sa_mode,
+                                         sb.data_ptr(), sb_mode, bias.data_ptr() if bias is not None else None,
+                                         out.data_ptr(), _ld(out) if M > 1 else max(N, 1), algo, ws_ptr, ws_bytes, st)
+    _lib.check(code, "l8_gemm_nt_ws")
     if user_out:
         _wrote_into(out)
     return out

@@ -21,7 +21,7 @@ def fp8(t):
     return t.to(torch.float8_e4m3fn)
 
 
-ALGOS = list(range(0, 15))
+ALGOS = list(range(0, 16))
 SHAPES_EXACT = [(1, 1, 16), (32, 32, 64), (256, 256, 128), (256, 256, 256), (300, 200, 144), (257, 513, 272),
                 (64, 1000, 48), (1000, 24, 208), (512, 768, 240)]
 
@@ -42,7 +42,7 @@ def test_exact_small_integer_operands(algo):
         assert torch.equal(out.cpu().double(), want), (algo, M, N, K)
 
 
-@pytest.mark.parametrize("algo", [0, 1, 2, 3, 11])
+@pytest.mark.parametrize("algo", [0, 1, 2, 3, 11, 15])
 def test_k_indexing_with_one_hot_operands(algo):
     # B[n] is one-hot at k = pi(n): C[m,n] = A[m, pi(n)] exactly, for any K (tails included)
     from lingua_amd import ops
@@ -127,3 +127,57 @@ def test_7b_shapes_vs_library_matmul_and_oracle_rows(mnk):
     rows = torch.arange(0, M, max(1, M // 48), device="cuda")[:48]
     want = oracle.gemm_nt(qa[rows].cpu().view(torch.uint8), qb.cpu().view(torch.uint8), sa[rows].cpu(), sb.cpu())
     assert rel_l2(out[rows], want) <= TOL
+
+
+# Shapes for which tile configuration 15 shares the K range of the last round's tiles out between workgroups (long K, tile
+# count a little above a multiple of the compute units; 256 compute units assumed, on other parts the same shapes
+# may run unsplit and the assertions hold all the same): 16 x 26 tiles with 64 K tiles (every XCD splits: 20 tail
+# tiles, 12 helpers with one or two pieces each), and 13 x 20 ragged tiles with 48 K tiles and a K tail (four XCDs
+# have one tail tile and split it, four have none).
+SHAPES_SHARED_K = [(4096, 6656, 8192), (3300, 5096, 6128)]
+SHAPES_SHARED_K_RANDOM = SHAPES_SHARED_K + [(11008, 4096, 16384)]  # + a 7B wgrad shape: three pieces per helper
+
+
+@pytest.mark.parametrize("mnk", SHAPES_SHARED_K)
+def test_shared_k_range_exact_and_repeatable(mnk):
+    # {-1, 0, 1} operands and power-of-two scales: every partial sum is exact in fp32, so the split product must
+    # equal the unsplit one and the true one bit for bit; two calls must agree bit for bit as well
+    from lingua_amd import _lib, ops
+    M, N, K = mnk
+    g = torch.Generator(device="cuda").manual_seed(K)
+    A = torch.randint(-1, 2, (M, K), generator=g, device="cuda").float()
+    B = torch.randint(-1, 2, (N, K), generator=g, device="cuda").float()
+    sa = torch.tensor([2.0 ** (i % 5 - 2) for i in range(M)], device="cuda").reshape(M, 1)
+    sb = torch.tensor([2.0 ** (i % 3) for i in range(N)], device="cuda").reshape(N, 1)
+    qa, qb = fp8(A), fp8(B)
+    out = ops.gemm_nt(qa, qb, sa, sb, algo=ops.GEMM_ALGO_SHARED_K)
+    torch.backends.cuda.matmul.allow_tf32 = False
+    want = ((A @ B.t()) * sa * sb.t()).to(torch.bfloat16)  # integer sums below 2^24: exact in fp32
+    assert torch.equal(out, want)
+    again = ops.gemm_nt(qa, qb, sa, sb, algo=ops.GEMM_ALGO_SHARED_K)
+    assert torch.equal(out, again)
+    # the entry point without a workspace never splits
+    plain = torch.empty_like(out)
+    code = _lib.load().l8_gemm_nt(qa.data_ptr(), qb.data_ptr(), M, N, K, K, K, sa.data_ptr(), ops.SCALE_ROW, sb.data_ptr(),
+                                  ops.SCALE_ROW, None, plain.data_ptr(), N, 0, torch.cuda.current_stream().cuda_stream)
+    _lib.check(code, "l8_gemm_nt")
+    assert torch.equal(out, plain)
+
+
+@pytest.mark.parametrize("mnk", SHAPES_SHARED_K_RANDOM)
+def test_shared_k_range_random_operands(mnk):
+    from lingua_amd import ops
+    M, N, K = mnk
+    g = torch.Generator().manual_seed(M)
+    qa, qb = random_fp8_bytes((M, K), g).cuda(), random_fp8_bytes((N, K), g).cuda()
+    sa = (torch.rand(M, 1, generator=g) + 0.5).cuda()
+    sb = (torch.rand(1, 1, generator=g) + 0.5).cuda()   # scalar scale on the B side, as in dgrad
+    A, B = qa.view(torch.float8_e4m3fn), qb.view(torch.float8_e4m3fn)
+    out = ops.gemm_nt(A, B, sa, sb, algo=ops.GEMM_ALGO_SHARED_K)
+    torch.backends.cuda.matmul.allow_tf32 = False
+    ref = ((A.float() * sa) @ (B.float() * sb).t()).to(torch.bfloat16)
+    assert rel_l2(out, ref) <= TOL
+    rows = torch.arange(0, M, M // 24, device="cuda")[:24]
+    want = oracle.gemm_nt(qa[rows].cpu(), qb.cpu(), sa[rows].cpu(), sb.cpu())
+    assert rel_l2(out[rows], want) <= TOL
+    assert torch.equal(out, ops.gemm_nt(A, B, sa, sb, algo=ops.GEMM_ALGO_SHARED_K))  # fixed order of the partial sums: repeatable bit for bit
