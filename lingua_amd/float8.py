@@ -64,6 +64,10 @@ class Fp8Config:
     # bf16 input: half the bytes held between forward and backward, the same
     # kernels and the same results (plain autograd.Function route only)
     save_fp8_input: bool = False
+    # keep the quantised copies of every weight (row-wise for forward, tensor-wise transposed for dgrad:
+    # 2 bytes per parameter) until the weight's version counter moves, so that micro-batches between two
+    # optimizer steps (gradient accumulation) and evaluation passes quantise each weight once
+    cache_weight_casts: bool = False
 
 
 config = Fp8Config()
@@ -89,7 +93,7 @@ def scale(t: torch.Tensor, amax_t: Optional[torch.Tensor] = None):
     ``[1,1]`` tensor-wise, ``[R,g]`` sub-row-wise -- every row in ``g`` equal
     column groups, each with a scale of its own, which is what the reference
     computes when tensor parallelism shards the reduction dimension over ``g``
-    ranks (lingua/float8.py:14-21, :86).  For the row-wise and sub-row-wise
+    ranks (lingua/float8.py:14-21, :86).
     The values of ``amax_t`` are used as given, as in the reference: a row-wise
     amax whose rows all hold the tensor's amax (what lingua/float8.py:115-118
     builds for dgrad) quantises tensor-wise, and an amax that is not the true
@@ -187,6 +191,60 @@ _bwd_cast = _LastCast()   # a -> (qat, sat)
 _fwd_tcast = _LastCast()  # a -> (qat, sat), made in forward when config.save_fp8_input
 
 
+class _WeightCasts:
+    """Quantised copies of weights, one entry per weight storage, valid while pointer, shape, strides, dtype,
+    version counter and stream are what they were (an optimizer step advances the version).  Used only with
+    ``config.cache_weight_casts``."""
+
+    def __init__(self):
+        self.entries = {}
+
+    def _slot(self, w):
+        if w.is_inference():
+            return None
+        key = _LastCast._key(w)
+        slot = self.entries.get(w.data_ptr())
+        if slot is None or slot["key"] != key:
+            slot = {"key": key, "w": w}
+            self.entries[w.data_ptr()] = slot
+        return slot
+
+    def rowwise(self, w):
+        slot = self._slot(w) if config.cache_weight_casts else None
+        if slot is not None and "row" in slot:
+            return slot["row"]
+        value = ops.cast_rowwise(w)
+        if slot is not None:
+            slot["row"] = value
+        return value
+
+    def tensorwise_t(self, w, amax_rows):
+        slot = self._slot(w) if config.cache_weight_casts else None
+        if slot is not None and "tw" in slot:
+            return slot["tw"]
+        value = ops.cast_tensorwise(w, ops.amax_reduce(amax_rows), transpose=True)
+        if slot is not None:
+            slot["tw"] = value
+        return value
+
+    def clear(self):
+        self.entries.clear()
+
+
+_weight_casts = _WeightCasts()
+
+
+def weight_cast_rowwise(w):
+    """``(q, scale, row amax)`` of a weight, row-wise (the forward operand, lingua/float8.py:87)."""
+    return _weight_casts.rowwise(w)
+
+
+def weight_cast_tensorwise_t(w, amax_rows):
+    """``(q [K,N], scale [1,1])`` of a weight [N,K], tensor-wise from its saved row amaxes and written
+    transposed (the dgrad operand, lingua/float8.py:111-118)."""
+    return _weight_casts.tensorwise_t(w, amax_rows)
+
+
 def clear_cast_memos() -> None:
     """Forget the shared activation casts.  The memos trust the tensor's version counter, exactly as
     autograd's check of saved tensors does: every PyTorch in-place op and every ``out=`` write of
@@ -196,6 +254,7 @@ def clear_cast_memos() -> None:
     _fwd_cast.clear()
     _bwd_cast.clear()
     _fwd_tcast.clear()
+    _weight_casts.clear()
 
 
 def linear_forward(a, b_t, bias, need_wgrad_stats: bool, gemm_algo: int):
@@ -215,7 +274,7 @@ def linear_forward(a, b_t, bias, need_wgrad_stats: bool, gemm_algo: int):
         qa, sa, _ = ops.cast_rowwise(a, col_amax=a_col_amax)
         if config.share_input_casts:
             _fwd_cast.put(a, (qa, sa, a_col_amax), b_t.data_ptr())
-    qb, sb, amax_b_t = ops.cast_rowwise(b_t)
+    qb, sb, amax_b_t = weight_cast_rowwise(b_t)
     out = ops.gemm_nt(qa, qb, sa, sb, bias, algo=gemm_algo)
     return out, amax_b_t, a_col_amax
 
@@ -251,8 +310,7 @@ def linear_backward(grad_out, a, b_t, amax_b_t, a_col_amax, need_a: bool, need_b
         # forward, quantised straight into the [K,N] layout dgrad multiplies with
         g_col_amax = torch.empty(grad_out.shape[1], dtype=torch.float32, device=grad_out.device) if fp8_wgrad else None
         qg, sg, _ = ops.cast_rowwise(grad_out, col_amax=g_col_amax)
-        amax_b = ops.amax_reduce(amax_b_t)
-        qb, sb = ops.cast_tensorwise(b_t, amax_b, transpose=True)
+        qb, sb = weight_cast_tensorwise_t(b_t, amax_b_t)
         grad_a = ops.gemm_nt(qg, qb, sg, sb, None, algo=gemm_algo)
     else:
         grad_a = None

@@ -48,14 +48,14 @@ class Fp8SwiGLUFn(torch.autograd.Function):
         else:
             x_col = torch.empty(x.shape[1], dtype=torch.float32, device=x.device) if need_x_col else None
             qx, sx, _ = ops.cast_rowwise(x, col_amax=x_col)
-        q1, s1, amax_w1 = ops.cast_rowwise(w1)
-        q3, s3, amax_w3 = ops.cast_rowwise(w3)
+        q1, s1, amax_w1 = f8.weight_cast_rowwise(w1)
+        q3, s3, amax_w3 = f8.weight_cast_rowwise(w3)
         h1 = ops.gemm_nt(qx, q1, sx, s1, None, algo=algo)
         h3 = ops.gemm_nt(qx, q3, sx, s3, None, algo=algo)
         del qx, q1, q3
         h_col = torch.empty(w2.shape[1], dtype=torch.float32, device=x.device) if fp8_wgrad and w2.requires_grad else None
         h, qh, sh, _ = ops.swiglu_cast_rowwise(h1, h3, want_h=w2.requires_grad, col_amax=h_col)
-        q2, s2, amax_w2 = ops.cast_rowwise(w2)
+        q2, s2, amax_w2 = f8.weight_cast_rowwise(w2)
         y = ops.gemm_nt(qh, q2, sh, s2, None, algo=algo)
 
         ctx.fp8_wgrad, ctx.gemm_algo = fp8_wgrad, algo
@@ -90,7 +90,7 @@ class Fp8SwiGLUFn(torch.autograd.Function):
 
         gy_col = torch.empty(D, dtype=torch.float32, device=dev) if fp8_wgrad and need_w2 else None
         qgy, sgy, _ = ops.cast_rowwise(gy, col_amax=gy_col)
-        qw2t, sw2t = ops.cast_tensorwise(w2, ops.amax_reduce(amax_w2), transpose=True)
+        qw2t, sw2t = f8.weight_cast_tensorwise_t(w2, amax_w2)
         dh = ops.gemm_nt(qgy, qw2t, sgy, sw2t, None, algo=algo)
         del qgy, qw2t
         if need_w2:
@@ -102,9 +102,9 @@ class Fp8SwiGLUFn(torch.autograd.Function):
         g1, g3, qg1, qg3, sg1, sg3 = ops.swiglu_bwd_cast_rowwise(dh, h1, h3, g1_col, g3_col)
         del dh
         if need_x:
-            qw1t, sw1t = ops.cast_tensorwise(w1, ops.amax_reduce(amax_w1), transpose=True)
+            qw1t, sw1t = f8.weight_cast_tensorwise_t(w1, amax_w1)
             gx = ops.gemm_nt(qg1, qw1t, sg1, sw1t, None, algo=algo)
-            qw3t, sw3t = ops.cast_tensorwise(w3, ops.amax_reduce(amax_w3), transpose=True)
+            qw3t, sw3t = f8.weight_cast_tensorwise_t(w3, amax_w3)
             gx += ops.gemm_nt(qg3, qw3t, sg3, sw3t, None, algo=algo)
         del qg1, qg3
         if need_w1 or need_w3:

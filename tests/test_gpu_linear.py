@@ -558,3 +558,50 @@ def test_selective_checkpointing_saves_the_fp8_product():
         assert torch.equal(a.view(torch.int16), b.view(torch.int16))
     for a, b in zip(full, plain):
         assert torch.equal(a.view(torch.int16), b.view(torch.int16))
+
+
+def test_weight_casts_kept_between_optimizer_steps():
+    """config.cache_weight_casts: micro-batches between two optimizer steps quantise each weight once (row-wise
+    for forward, tensor-wise transposed for dgrad); an in-place update of the weight is seen; same bits."""
+    from lingua_amd import Fp8Linear, float8, ops
+    torch.manual_seed(8)
+    lin = Fp8Linear(256, 384, bias=False, device="cuda", dtype=torch.bfloat16)
+    xs = [seeded_bf16((48, 256), seed=30 + i).cuda().requires_grad_(True) for i in range(2)]
+    g = seeded_bf16((48, 384), std=0.02, seed=33).cuda()
+
+    def micro_batches(cache):
+        old = float8.config.cache_weight_casts
+        float8.config.cache_weight_casts = cache
+        float8.clear_cast_memos()
+        rec = []
+        ops.kernel_timer = rec
+        try:
+            outs = []
+            for x in xs:
+                x.grad = None
+                lin.weight.grad = None
+                y = lin(x)
+                y.backward(g)
+                outs += [y.detach(), x.grad.clone(), lin.weight.grad.clone()]
+            counts = (sum(1 for r in rec if r[0] == "cast_rowwise"), sum(1 for r in rec if r[0] == "cast_tensorwise_t"))
+            del rec[:]
+            with torch.no_grad():
+                lin.weight.mul_(0.5)       # the optimizer step
+            y = lin(xs[0])
+            outs.append(y.detach())
+            after_step = sum(1 for r in rec if r[0] == "cast_rowwise")
+        finally:
+            ops.kernel_timer = None
+            float8.config.cache_weight_casts = old
+            float8.clear_cast_memos()
+            with torch.no_grad():
+                lin.weight.mul_(2.0)
+        return outs, counts, after_step
+
+    plain, counts_plain, again_plain = micro_batches(False)
+    cached, counts_cached, again_cached = micro_batches(True)
+    assert counts_plain == (6, 2), counts_plain    # per micro-batch: x, W, grad row-wise; W tensor-wise transposed
+    assert counts_cached == (5, 1), counts_cached  # the weight once in each layout
+    assert again_plain == 2 and again_cached == 2  # a changed weight is quantised again
+    for a, b in zip(plain, cached):
+        assert torch.equal(a.view(torch.int16), b.view(torch.int16))
