@@ -35,7 +35,7 @@ PEAK_HBM_GBPS = 8000.0                       # MI355X HBM3E, published
 # times each: forward 1.527 GB, dgrad 1.234 GB, wgrad 1.435 GB (algorithmic: 473 / 360 / 338 MB).  A counter run
 # cannot share a process with the timed steps (it slows the kernels by ~8 %), so the figure is carried over from
 # the profile of this same kernel and shapes and named as such in the JSON line.
-GEMM_TRAFFIC_BYTES = 1_399_000_000
+GEMM_TRAFFIC_BYTES = 1_370_000_000
 
 
 def parse():
@@ -450,7 +450,7 @@ def main():
                                  "frac_hbm": round(gbps / PEAK_HBM_GBPS, 4)}
         n, ms, work = agg["gemm_nt"]
         achieved = work / (ms * 1e-3) / 1e12
-        roofline = {"kernel": "gemm_nt_stream_kernel<4,false> (fp8 e4m3 NT GEMM, 2*16384*4096*11008 flop per launch; forward, dgrad and wgrad products)",
+        roofline = {"kernel": "gemm_nt_stream_kernel<4,false,false> (fp8 e4m3 NT GEMM, 2*16384*4096*11008 flop per launch; forward, dgrad and wgrad products)",
                     "bound": "mfma", "achieved": round(achieved, 1), "peak": PEAK_FP8_TFLOPS, "unit": "TFLOP/s",
                     "frac": round(achieved / PEAK_FP8_TFLOPS, 4), "traffic": GEMM_TRAFFIC_BYTES,
                     "traffic_unit": "bytes per launch, mean of the step's three products (algorithmic: 390 MB); from "
