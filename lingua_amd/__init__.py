@@ -3,6 +3,7 @@ from .float8 import (  # noqa: F401
     EPS,
     Fp8Linear,
     Fp8LinearFn,
+    clear_cast_memos,
     config,
     convert_linears_to_fp8,
     matmul,
@@ -14,6 +15,7 @@ __all__ = [
     "EPS",
     "Fp8Linear",
     "Fp8LinearFn",
+    "clear_cast_memos",
     "config",
     "convert_linears_to_fp8",
     "matmul",
