@@ -148,6 +148,11 @@ int l8_gemm_nt_ws(const void *A, const void *B, int64_t M, int64_t N, int64_t K,
                   const void *bias, void *C, int64_t ldc, int algo,
                   void *workspace, int64_t workspace_bytes, void *stream);
 int64_t l8_gemm_workspace(void);
+/* Testing aid for the exchange above (no counterpart in the reference): how many times (about a microsecond
+ * each) a workgroup polls for another's partial sums before it gives up and fills its tile with NaN instead
+ * of waiting for ever.  Default 262144; 0 makes every shared tile give up at once, which is how the tests
+ * reach that path without hanging anything.  Process-wide. */
+int l8_gemm_set_wait_limit(int polls);
 
 /* SwiGLU gate fused with the row-wise cast of the w2 input.
  * Replaces `F.silu(self.w1(x)) * self.w3(x)` of lingua/transformer.py:469-471 (two bf16

@@ -69,6 +69,7 @@ struct GemmArgs {
   uint32_t *sk_flags;
   float *sk_partials;
   uint32_t sk_epoch;  // value that marks a flag as set in THIS launch (never 0; flags are never cleared)
+  int sk_wait_limit;  // polls of a flag before the waiting workgroup gives up and poisons its tile
 };
 
 typedef __attribute__((address_space(3))) void *lds_ptr_t;
@@ -922,7 +923,7 @@ __global__ __launch_bounds__(256) void gemm_nt_stream_kernel(const GemmArgs p) {
   // that never comes poisons the tile with a NaN instead of hanging the GPU.
   [[maybe_unused]] auto wait_partial = [&](int slot) -> bool {
 #pragma unroll 1
-    for (int spin = 0; spin < (1 << 18); ++spin) {
+    for (int spin = 0; spin < p.sk_wait_limit; ++spin) {
       const uint32_t f = __hip_atomic_load(p.sk_flags + slot, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
       if ((uint32_t)__builtin_amdgcn_readfirstlane((int)f) == p.sk_epoch) return true;
       __builtin_amdgcn_s_sleep(32);
@@ -1171,6 +1172,14 @@ static int pick_algo(int64_t M, int64_t N, int64_t K) {
 // flags (one 4-byte word per workgroup, first 4 KiB) + one fp32 256x256 tile per workgroup of a persistent launch
 constexpr int64_t kSkMaxGrid = 1024, kSkFlagBytes = kSkMaxGrid * 4, kSkTileBytes = 256 * 256 * 4;
 static std::atomic<uint32_t> g_sk_epoch{0};
+// polls (about a microsecond each) an owner spends on a helper's flag before it gives up: a third of a second
+static std::atomic<int> g_sk_wait_limit{1 << 18};
+
+extern "C" int l8_gemm_set_wait_limit(int polls) {
+  L8_REQUIRE(polls >= 0, "l8_gemm_set_wait_limit: negative limit");
+  g_sk_wait_limit = polls;
+  return L8_OK;
+}
 
 extern "C" int64_t l8_gemm_workspace(void) {
   const int64_t cus8 = (num_cus() / 8) * 8;
@@ -1232,6 +1241,7 @@ static int gemm_nt_impl(const void *A, const void *B, int64_t M, int64_t N, int6
   p.sk_flags = nullptr;
   p.sk_partials = nullptr;
   p.sk_epoch = 0;
+  p.sk_wait_limit = 0;
   p.dbg = nullptr;
   if (L8_GEMM_PROF && al.persistent) {
     p.dbg = (uint64_t *)bias;
@@ -1281,6 +1291,7 @@ static int gemm_nt_impl(const void *A, const void *B, int64_t M, int64_t N, int6
       uint32_t e = ++g_sk_epoch;
       if (e == 0) e = ++g_sk_epoch;  // 0 is what an untouched flag holds
       p.sk_epoch = e;
+      p.sk_wait_limit = g_sk_wait_limit;
     }
   }
   hipLaunchKernelGGL(fn, dim3((unsigned)grid), dim3(al.threads), al.lds, (hipStream_t)stream, p);

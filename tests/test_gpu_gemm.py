@@ -181,3 +181,31 @@ def test_shared_k_range_random_operands(mnk):
     want = oracle.gemm_nt(qa[rows].cpu(), qb.cpu(), sa[rows].cpu(), sb.cpu())
     assert rel_l2(out[rows], want) <= TOL
     assert torch.equal(out, ops.gemm_nt(A, B, sa, sb, algo=ops.GEMM_ALGO_SHARED_K))  # fixed order of the partial sums: repeatable bit for bit
+
+
+def test_shared_k_range_gives_up_instead_of_hanging():
+    # With a wait limit of zero polls an owner never sees its helper's partial sums: its tile must come out as
+    # NaN (never as a wrong number), the kernel must still finish, and the next call with the normal limit is right.
+    from lingua_amd import _lib, ops
+    M, N, K = SHAPES_SHARED_K[0]
+    g = torch.Generator(device="cuda").manual_seed(3)
+    A = torch.randint(-1, 2, (M, K), generator=g, device="cuda").float()
+    B = torch.randint(-1, 2, (N, K), generator=g, device="cuda").float()
+    one = torch.ones(1, 1, device="cuda")
+    qa, qb = fp8(A), fp8(B)
+    want = (A @ B.t()).to(torch.bfloat16)
+    lib = _lib.load()
+    _lib.check(lib.l8_gemm_set_wait_limit(0), "l8_gemm_set_wait_limit")
+    try:
+        out = ops.gemm_nt(qa, qb, one, one, algo=ops.GEMM_ALGO_SHARED_K)
+        torch.cuda.synchronize()
+    finally:
+        _lib.check(lib.l8_gemm_set_wait_limit(1 << 18), "l8_gemm_set_wait_limit")
+    bad = torch.isnan(out)
+    assert torch.equal(out[~bad], want[~bad])           # what is not poisoned is right
+    if torch.cuda.get_device_properties(0).multi_processor_count == 256:
+        tiles = bad.reshape(M // 256, 256, N // 256, 256).permute(0, 2, 1, 3).reshape(-1, 256 * 256)
+        n_bad = int(tiles.all(dim=1).sum())
+        assert n_bad == int(tiles.any(dim=1).sum())      # whole tiles, nothing partial
+        assert n_bad == 8 * 20                           # the 20 tail tiles of each XCD
+    assert torch.equal(ops.gemm_nt(qa, qb, one, one, algo=ops.GEMM_ALGO_SHARED_K), want)
