@@ -863,7 +863,8 @@ __global__ __launch_bounds__(256) void gemm_nt_stream_kernel(const GemmArgs p) {
           const int got0 = __builtin_amdgcn_update_dpp(0, give0, 0xB1, 0xF, 0xF, true);
           const int got1 = __builtin_amdgcn_update_dpp(0, give1, 0xB1, 0xF, 0xF, true);
           const v4i out = par ? v4i{got0, got1, o[1][0], o[1][1]} : v4i{o[0][0], o[0][1], got0, got1};
-          __builtin_amdgcn_raw_buffer_store_b128(out, rsC, c_voff, (row + e2) * ldc2, 2 /* streaming */);
+          if (L8_GEMM_DIAG != 3 && !(L8_GEMM_DIAG == 8 && (qd & 1)))  // experiments: no stores (3), half of them (8)
+            __builtin_amdgcn_raw_buffer_store_b128(out, rsC, c_voff, (row + e2) * ldc2, 2 /* streaming */);
           // one row pair at a time: left free, the scheduler reads a hundred accumulator registers ahead and the
           // register pressure of this conversion makes the allocator spill values the K loop uses in every trip
           __builtin_amdgcn_sched_barrier(0);
