@@ -262,10 +262,11 @@ def measure_llama1b(torch, dev, steps, warmup, fused_too=True):
     dt = timed(model)
     fused_dt = None
     if fused_too:
-        # same weights, gate fused into the casts and norms that hand their output over quantised
+        # same weights, gate fused into the casts, norms that hand their output over quantised, one product for wq/wk/wv
         from lingua_amd.norm import fuse_rmsnorm
+        from lingua_amd.qkv import fuse_qkv
         from lingua_amd.swiglu import fuse_feed_forward
-        fused_dt = timed(fuse_rmsnorm(fuse_feed_forward(model)))
+        fused_dt = timed(fuse_qkv(fuse_rmsnorm(fuse_feed_forward(model))))
     fpt = llama_flops_per_token(LLAMA_1B["n_layers"], LLAMA_1B["dim"], LLAMA_1B["ffn_dim"], LLAMA_1B["vocab"], S)
     fp8_flop = 25 * 3 * (4 * 2 * B * S * 2048 * 2048 + 3 * 2 * B * S * 2048 * 8192)
     res = {"value": round(B * S / dt, 1), "unit": "tokens/s", "ms_per_step": round(dt * 1e3, 3), "steps": steps, "warmup": warmup,

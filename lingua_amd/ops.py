@@ -91,7 +91,10 @@ def cast_rowwise(x: torch.Tensor, col_amax: Optional[torch.Tensor] = None, want_
         q = out_q if out_q is not None else torch.empty((R, C), dtype=torch.float8_e4m3fn, device=x.device)
         if q.dtype != torch.float8_e4m3fn or tuple(q.shape) != (R, C) or q.device != x.device or (q.numel() and q.stride(1) != 1):
             raise RuntimeError("cast_rowwise: out_q must be an e4m3fn [R,C] tensor on x's device with unit column stride")
-    scale = torch.empty((R, 1), dtype=torch.float32, device=x.device)
+    if out_scale is not None and (out_scale.dtype != torch.float32 or tuple(out_scale.shape) != (R, 1) or out_scale.device != x.device):
+        raise RuntimeError("cast_rowwise: out_scale must be fp32 [R,1] on x's device")
+    scale_direct = out_scale is not None and (R <= 1 or out_scale.stride(0) == 1)  # the kernel writes a dense vector
+    scale = out_scale if scale_direct else torch.empty((R, 1), dtype=torch.float32, device=x.device)
     amax = torch.empty((R, 1), dtype=torch.bfloat16, device=x.device)
     if col_amax is not None and (col_amax.dtype != torch.float32 or col_amax.numel() != C or not col_amax.is_contiguous()):
         raise RuntimeError("cast_rowwise: col_amax must be a contiguous fp32 tensor with C elements")
@@ -108,9 +111,9 @@ def cast_rowwise(x: torch.Tensor, col_amax: Optional[torch.Tensor] = None, want_
     _lib.check(code, "l8_cast_rowwise")
     if out_q is not None and want_q:
         _wrote_into(out_q)
-    if out_scale is not None:
-        if out_scale.dtype != torch.float32 or tuple(out_scale.shape) != (R, 1):
-            raise RuntimeError("cast_rowwise: out_scale must be fp32 [R,1]")
+    if scale_direct:
+        _wrote_into(out_scale)
+    elif out_scale is not None:
         scale = out_scale.copy_(scale)
     return q, scale, amax
 
