@@ -397,19 +397,19 @@ def main():
             y.backward(gy)
         return step
 
-    def timed(module, records):
+    def timed(module, records, names=None):
         step = make_step(module)
         for _ in range(args.warmup):
             step()
         torch.cuda.synchronize()
-        ops.kernel_timer = records
+        ops.kernel_timer, ops.kernel_timer_names = records, names
         torch.cuda.synchronize()
         t0 = time.perf_counter()
         for _ in range(args.steps):
             step()
         torch.cuda.synchronize()
         elapsed = time.perf_counter() - t0
-        ops.kernel_timer = None
+        ops.kernel_timer, ops.kernel_timer_names = None, None
         return elapsed
 
     def sustained(module, seconds):
@@ -426,8 +426,15 @@ def main():
                 return {"value": round(STEP_FLOP * n / el / 1e12, 2), "unit": "TFLOP/s", "steps": n, "seconds": round(el, 2),
                         "ms_per_step": round(el / n * 1e3, 4)}
 
+    # Inside the timed steps only the GEMM launches (the roofline kernel) are bracketed by events: a pair of events
+    # around every launch of the step costs 2.6 % of the step's time (measured), around the nine GEMMs 0.8 %.  The
+    # cast kernels' table comes from a second, untimed-for-`value` pass with every launch bracketed.
     records = None if args.no_kernel_timing else []
-    dt = timed(mlp, records)
+    dt = timed(mlp, records, {"gemm_nt"})
+    if records is not None:
+        cast_records = []
+        timed(mlp, cast_records)
+        records += [r for r in cast_records if r[0] != "gemm_nt"]
 
     ms_per_step = dt / args.steps * 1e3
     tflops = STEP_FLOP / (dt / args.steps) / 1e12

@@ -17,7 +17,10 @@ SCALE_ROW = 1
 # appends (kernel name, start event, end event, algorithmic work) where the
 # events are recorded on the stream the kernel runs on.  Work is flop for the
 # GEMM and compulsory bytes for the casts.  None (the default) records nothing.
+# `kernel_timer_names` (a set of kernel names, or None for all) limits the recording: every pair of events costs
+# the stream a little, which a caller timing a whole step may not want to pay for every launch.
 kernel_timer = None
+kernel_timer_names = None
 
 
 class _timed:
@@ -34,7 +37,7 @@ class _timed:
         if self.dev.index is not None and self.dev.index != cur:
             self.prev = cur
             torch.cuda.set_device(self.dev)
-        if kernel_timer is not None:
+        if kernel_timer is not None and (kernel_timer_names is None or self.name in kernel_timer_names):
             self.ev = (torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True))
             self.ev[0].record(torch.cuda.current_stream(self.dev))
 
