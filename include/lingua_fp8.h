@@ -148,6 +148,10 @@ int l8_gemm_nt_ws(const void *A, const void *B, int64_t M, int64_t N, int64_t K,
                   const void *bias, void *C, int64_t ldc, int algo,
                   void *workspace, int64_t workspace_bytes, void *stream);
 int64_t l8_gemm_workspace(void);
+/* Host arithmetic only: the number of XCDs (0..8) that would share the K range of their last round's tiles out
+ * under tile configuration 15, for this problem on a part with `compute_units` compute units (256 on MI355X).
+ * 0 = configuration 15 behaves exactly like configuration 12.  No counterpart in the reference. */
+int l8_gemm_shares_k(int64_t M, int64_t N, int64_t K, int compute_units);
 /* Testing aid for the exchange above (no counterpart in the reference): how many times (about a microsecond
  * each) a workgroup polls for another's partial sums before it gives up and fills its tile with NaN instead
  * of waiting for ever.  Default 262144; 0 makes every shared tile give up at once, which is how the tests

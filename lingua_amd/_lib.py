@@ -32,6 +32,7 @@ SIGNATURES = {
     "l8_gemm_nt_ws": [_p, _p, _i64, _i64, _i64, _i64, _i64, _p, _int, _p, _int, _p, _p, _i64, _int, _p, _i64, _p],
     "l8_gemm_workspace": [],
     "l8_gemm_set_wait_limit": [_int],
+    "l8_gemm_shares_k": [_i64, _i64, _i64, _int],
     "l8_swiglu_cast_rowwise": [_p, _p, _i64, _i64, _i64, _i64, _p, _i64, _p, _i64, _p, _p, _p, _p, _i64, _p],
     "l8_swiglu_workspace": [_i64, _i64],
     "l8_swiglu_bwd_cast_rowwise": [_p, _p, _p, _i64, _i64, _i64, _i64, _i64, _p, _p, _i64, _p, _p, _i64, _p, _p, _p, _p,

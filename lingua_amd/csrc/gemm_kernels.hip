@@ -1196,6 +1196,18 @@ static bool sk_pays(int64_t cnt, int64_t W, int64_t KT) {
   return n_rounds > 0 && r > 0 && l_help >= kSkMinSaved;
 }
 
+// Host arithmetic only (no GPU needed): on a part with `compute_units` compute units, how many of the 8 XCDs would
+// share out the K range of their last round's tiles under tile configuration 15 for this problem.
+extern "C" int l8_gemm_shares_k(int64_t M, int64_t N, int64_t K, int compute_units) {
+  L8_REQUIRE(M >= 0 && N >= 0 && K >= 0 && compute_units >= 8, "l8_gemm_shares_k: bad argument");
+  const int64_t nblocks = ((M + 255) / 256) * ((N + 255) / 256), KT = (K + 127) / 128;
+  const int64_t cus8 = (compute_units / 8) * 8, want = (nblocks + 7) / 8 * 8;
+  int64_t grid = want < cus8 ? want : cus8;
+  if (grid < 8) grid = 8;
+  const int64_t W = grid / 8, q = nblocks / 8, rem = nblocks % 8;
+  return (int)((sk_pays(q + 1, W, KT) ? rem : 0) + (sk_pays(q, W, KT) ? 8 - rem : 0));
+}
+
 static int gemm_nt_impl(const void *A, const void *B, int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldb,
                         const float *sa, int sa_mode, const float *sb, int sb_mode, const void *bias, void *C,
                         int64_t ldc, int algo, void *workspace, int64_t workspace_bytes, void *stream) {

@@ -162,3 +162,53 @@ def test_custom_op_fake_kernels_on_meta_tensors():
     assert ga.shape == a.shape and gb.shape == w.shape and gbias.shape == (48,)
     ga, gb, gbias = torch.ops.lingua_amd.fp8_linear_bwd(out, a, w, amax_w, col, False, True, False, True, 0)
     assert ga.numel() == 0 and gb.shape == w.shape and gbias.numel() == 0
+
+
+def test_which_problems_share_the_k_range_of_their_last_round():
+    """Host-side decision of tile configuration 15 (no GPU needed): the K range of the last round's tiles is shared
+    out only where the exchange of partial sums pays, and the split the rule describes covers every (tile, K tile)
+    of the tail exactly once with every owner waiting only for a workgroup with a lower number."""
+    lib = _lib.load()
+    cus = 256
+    # the step's three products on 256 compute units: only the K = 16384 one (688 tiles, 2.69 rounds) splits
+    assert lib.l8_gemm_shares_k(11008, 4096, 16384, cus) == 8
+    assert lib.l8_gemm_shares_k(4096, 11008, 16384, cus) == 8
+    assert lib.l8_gemm_shares_k(16384, 11008, 4096, cus) == 0      # K loop too short to pay for the exchange
+    assert lib.l8_gemm_shares_k(16384, 4096, 11008, cus) == 0      # 1024 tiles: four full rounds
+    assert lib.l8_gemm_shares_k(4096, 6656, 8192, cus) == 8
+    assert lib.l8_gemm_shares_k(3300, 5096, 6128, cus) == 4        # four XCDs have a tail tile, four have none
+    assert lib.l8_gemm_shares_k(1024, 1024, 16384, cus) == 0       # less than one round: nothing to share
+    assert lib.l8_gemm_shares_k(16384, 4096, 11008, 4) < 0         # bad argument
+
+    def split(cnt, W, KT, write=8, fix=4, least=16):
+        rounds, r = divmod(cnt, W)
+        if rounds == 0 or r == 0:
+            return None
+        helpers = W - r
+        m = (r + helpers - 1) // helpers
+        piece = (KT + fix - m * write) // (m + 1)
+        return None if piece < least else (r, helpers, KT - piece)
+
+    for W in (1, 2, 5, 16, 32, 38):
+        for cnt in range(1, 3 * W + 1):
+            for KT in (1, 20, 47, 48, 64, 100, 128, 500):
+                s = split(cnt, W, KT)
+                got = lib.l8_gemm_shares_k(256 * 8 * cnt, 256, 128 * KT, 8 * W)
+                assert got == (8 if s else 0), (cnt, W, KT)
+                if not s:
+                    continue
+                r, helpers, cut = s
+                assert 0 < cut < KT
+                cover = {}
+                for loc in range(W):
+                    if loc < helpers:                      # helper: K tiles cut.. of tiles loc, loc + helpers, ...
+                        for tt in range(loc, r, helpers):
+                            for k in range(cut, KT):
+                                assert (tt, k) not in cover
+                                cover[(tt, k)] = loc
+                    else:                                  # owner of tile loc - helpers: K tiles 0..cut-1
+                        for k in range(cut):
+                            assert (loc - helpers, k) not in cover
+                            cover[(loc - helpers, k)] = loc
+                assert len(cover) == r * KT
+                assert all(cover[(tt, KT - 1)] < cover[(tt, 0)] for tt in range(r))
