@@ -4,6 +4,7 @@
 built ahead of time, in-tree; nothing compiles at import or at first call.
 """
 import os
+import re
 import subprocess
 import sys
 from concurrent.futures import ThreadPoolExecutor
@@ -29,15 +30,40 @@ HIPCC_FLAGS = [
 
 
 def _run(cmd, verbose):
+    """Runs one hipcc command; returns the register / scratch figures of the kernels it compiled
+    ({mangled name: {"VGPRs": n, "AGPRs": n, "ScratchSize": bytes per lane, "VGPRs Spill": n, "SGPRs Spill": n}})."""
     if verbose:
         print(" ".join(cmd), flush=True)
     res = subprocess.run(cmd, capture_output=True, text=True)
-    # the host pass of hipcc does not know the packed-fp32 feature and says so; that is harmless
-    err = "\n".join(l for l in res.stderr.splitlines() if "packed-fp32-ops" not in l)
+    usage, cur, rest = {}, None, []
+    for line in res.stderr.splitlines():
+        if "packed-fp32-ops" in line:
+            continue  # the host pass of hipcc does not know the packed-fp32 feature and says so; that is harmless
+        if "[-Rpass-analysis=kernel-resource-usage]" in line:
+            m = re.search(r"Function Name: (\S+)", line)
+            if m:
+                cur = usage.setdefault(m.group(1), {})
+            m = re.search(r"remark:\s+(VGPRs Spill|SGPRs Spill|ScratchSize|VGPRs|AGPRs)(?: \[[^\]]*\])?: (\d+)", line)
+            if m and cur is not None:
+                cur[m.group(1)] = int(m.group(2))
+            continue
+        rest.append(line)
+    err = "\n".join(rest)
     if res.returncode != 0:
         raise RuntimeError(f"hipcc failed ({res.returncode}):\n{err}")
     if verbose and err.strip():
         print(err, file=sys.stderr)
+    return usage
+
+
+def _check_usage(usage) -> None:
+    """The persistent GEMM kernel runs at the edge of the register file: a source change that makes the allocator
+    spill (or leaves loop state in private memory, which turns every panel load into a loop over lanes) costs a
+    third of its speed and no test would notice.  Such a build fails here instead."""
+    bad = [f"{name}: {u}" for name, u in usage.items()
+           if "gemm_nt_stream_kernel" in name and (u.get("ScratchSize", 0) or u.get("VGPRs Spill", 0))]
+    if bad:
+        raise RuntimeError("the persistent GEMM kernel must not use scratch memory:\n  " + "\n  ".join(bad))
 
 
 def build(verbose: bool = False) -> str:
@@ -45,9 +71,15 @@ def build(verbose: bool = False) -> str:
     hipcc = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
     os.makedirs(OBJ_DIR, exist_ok=True)
     objs = [os.path.join(OBJ_DIR, os.path.splitext(src)[0] + ".o") for src in SOURCES]
-    cmds = [[hipcc, *HIPCC_FLAGS, "-c", os.path.join(CSRC, src), "-o", obj] for src, obj in zip(SOURCES, objs)]
+    cmds = [[hipcc, *HIPCC_FLAGS, *(["-Rpass-analysis=kernel-resource-usage"] if src.endswith(".hip") else []),
+             "-c", os.path.join(CSRC, src), "-o", obj] for src, obj in zip(SOURCES, objs)]
     with ThreadPoolExecutor(max_workers=min(len(cmds), os.cpu_count() or 1)) as pool:
-        list(pool.map(lambda c: _run(c, verbose), cmds))
+        usages = list(pool.map(lambda c: _run(c, verbose), cmds))
+    usage = {k: v for u in usages for k, v in u.items()}
+    with open(os.path.join(OBJ_DIR, "resource_usage.txt"), "w") as f:
+        for name in sorted(usage):
+            f.write(f"{name} {usage[name]}\n")
+    _check_usage(usage)
     _run([hipcc, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", LIB_PATH, *objs], verbose)
     return LIB_PATH
 

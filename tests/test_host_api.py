@@ -212,3 +212,15 @@ def test_which_problems_share_the_k_range_of_their_last_round():
                             cover[(loc - helpers, k)] = loc
                 assert len(cover) == r * KT
                 assert all(cover[(tt, KT - 1)] < cover[(tt, 0)] for tt in range(r))
+
+
+def test_build_refuses_a_persistent_gemm_kernel_that_uses_scratch():
+    from lingua_amd import build
+    ok = {"_ZN2l821gemm_nt_stream_kernelILi4ELb0ELb0EEEvNS_8GemmArgsE": {"VGPRs": 158, "AGPRs": 256, "ScratchSize": 0, "VGPRs Spill": 0},
+          "_ZN2l814gemm_nt_kernelILi2ELi2ELi4ELi4ELi5ELi8ELi0EEEvNS_8GemmArgsE": {"ScratchSize": 36, "VGPRs Spill": 8}}
+    build._check_usage(ok)   # the one-workgroup-per-tile kernels may spill outside their K loop
+    for field in ("ScratchSize", "VGPRs Spill"):
+        bad = {k: dict(v) for k, v in ok.items()}
+        bad["_ZN2l821gemm_nt_stream_kernelILi4ELb0ELb0EEEvNS_8GemmArgsE"][field] = 12
+        with pytest.raises(RuntimeError):
+            build._check_usage(bad)
