@@ -96,6 +96,10 @@ L8_DEV __amdgpu_buffer_rsrc_t make_rsrc(const void *p, uint32_t bytes) {
 #ifndef L8_STRADDLE
 #define L8_STRADDLE 2
 #endif
+// groups (of one MFMA each) of a half trip over which the persistent kernel issues the half's LDS reads
+#ifndef L8_READ_GROUPS
+#define L8_READ_GROUPS 13
+#endif
 // L8_GEMM_PROF (compile-time, never set in the shipped build): the persistent kernel takes the `bias` pointer for
 // a buffer of 16 x uint64 per workgroup and records wall-clock ticks (100 MHz) at its start, after the prologue
 // and at its end, and shader-clock cycles spent in the K loops and in the C-tile stores.
@@ -963,34 +967,48 @@ __global__ __launch_bounds__(256) void gemm_nt_stream_kernel(const GemmArgs p) {
   int s0 = 0;  // ring slot of the A panel of the K tile being multiplied
   // WAIT = the count of the wait in front of the barrier: everything older than the WAIT youngest requests must
   // have landed.
+  // A wave issues in order and the matrix cores want an MFMA every 64 cycles, about a dozen issue slots: a group
+  // that carries more than that leaves them idle.  So nothing but its MFMA, LDS reads and panel loads goes into a
+  // group: the fragment addresses of a half are formed in the middle of the half before (ad_a for the first half,
+  // ad_b for the second), and the LDS reads of a half are all issued in its first RD groups, so that the wait for
+  // them at the end of the half (barrier, loop top) finds them landed.
+  constexpr int RD = L8_READ_GROUPS, G_ADDR = 8;
+  static_assert(RD >= NF / 2 && RD <= S1 && RD <= S2 - STRADDLE && G_ADDR < S1, "group layout");
+  uint32_t ad_a[4], ad_b[4];
+  frag_addrs(0, 1, 1, ad_a);
   auto trip = [&](auto wait_tag) {
     constexpr int WAIT = decltype(wait_tag)::value;
     const int slot_u1 = wrap(s0 + R - 1);
-    frag_addrs(s0, wrap(s0 + 1), 1, ad);
 #pragma unroll
     for (int i = 0; i < S1; ++i) {
       mma_one(af0, bf0, i);
+      if (i < RD) {
 #pragma unroll
-      for (int f = (NF * i) / S1; f < (NF * (i + 1)) / S1; ++f) read_one(ad, af1, bf1, f);
+        for (int f = (NF * i) / RD; f < (NF * (i + 1)) / RD; ++f) read_one(ad_a, af1, bf1, f);
+      }
 #pragma unroll
       for (int j = (NL * i) / S1; j < (NL * (i + 1)) / S1; ++j) load_one(false, slot_u1, j);
+      if (i == G_ADDR) frag_addrs(wrap(s0 + 2), wrap(s0 + 3), 0, ad_b);
       __builtin_amdgcn_sched_barrier(0);
     }
     L8_WAIT_VM_LGKM0(WAIT);
     asm volatile("" ::: "memory");
     __builtin_amdgcn_s_barrier();
     asm volatile("" ::: "memory");
-    frag_addrs(wrap(s0 + 2), wrap(s0 + 3), 0, ad);
 #pragma unroll
     for (int i = 0; i < S2; ++i) {
       if (i < STRADDLE) mma_one(af0, bf0, S1 + i);
       else mma_one(af1, bf1, i - STRADDLE);
-      if (i >= STRADDLE) {
+      if (i >= STRADDLE && i - STRADDLE < RD) {
 #pragma unroll
-        for (int f = (NF * (i - STRADDLE)) / SR; f < (NF * (i - STRADDLE + 1)) / SR && f < NF; ++f) read_one(ad, af0, bf0, f);
+        for (int f = (NF * (i - STRADDLE)) / RD; f < (NF * (i - STRADDLE + 1)) / RD; ++f) read_one(ad_b, af0, bf0, f);
       }
 #pragma unroll
       for (int j = (NL * i) / S2; j < (NL * (i + 1)) / S2; ++j) load_one(true, s0, j);
+      if (i == STRADDLE + G_ADDR) {
+        const int s_next = wrap(s0 + 2);
+        frag_addrs(s_next, wrap(s_next + 1), 1, ad_a);
+      }
       __builtin_amdgcn_sched_barrier(0);
     }
     ld_advance();
