@@ -116,6 +116,24 @@ def cpu_baseline(torch, sample_tokens):
         rt.linear_forward(x1, w1c)
         reps.append(time.perf_counter() - t0)
     c1 = sorted(reps[1:])[1]   # median of three after one warm-up
+    # configs[1]: Llama-1B-shaped SwiGLU MLP forward, 32768 tokens, one repetition
+    x2 = torch.randn(32768, 2048, generator=g).to(torch.bfloat16)
+    v1 = (torch.randn(8192, 2048, generator=g) * 0.02).to(torch.bfloat16)
+    v3 = (torch.randn(8192, 2048, generator=g) * 0.02).to(torch.bfloat16)
+    v2 = (torch.randn(2048, 8192, generator=g) * 0.02).to(torch.bfloat16)
+    t0 = time.perf_counter()
+    rt.linear_forward(torch.nn.functional.silu(rt.linear_forward(x2, v1)) * rt.linear_forward(x2, v3), v2)
+    c2 = time.perf_counter() - t0
+    del x2, v1, v2, v3
+    # configs[3]: the 4096 -> 11008 linear on the outlier-stress activations, row-wise and tensor-wise, one repetition
+    from workloads import outlier_stress_input, seeded_bf16
+    x4, _, _ = outlier_stress_input(rows=TOKENS, cols=DIM, seed=0)
+    w4 = seeded_bf16((FFN, DIM), 0.02, seed=1)
+    t0 = time.perf_counter()
+    rt.linear_forward(x4, w4)
+    rt.matmul(x4, x4.abs().amax().reshape(1, 1), w4, w4.abs().amax().reshape(1, 1))
+    c4 = time.perf_counter() - t0
+    del x4, w4
     return {
         "value": round(flop / dt / 1e12, 4),
         "unit": "TFLOP/s",
@@ -125,6 +143,11 @@ def cpu_baseline(torch, sample_tokens):
                   f"(PyTorch CPU ops: amax/clamp/div/reciprocal/mul/to(float8_e4m3fn), dequantise, fp32 matmul, bf16)",
         "config1_linear_forward": {"value": round(2 * 4096 * 2048 * 2048 / c1 / 1e12, 4), "unit": "TFLOP/s",
                                    "ms": round(c1 * 1e3, 2), "sample": "x [4096,2048] @ W [2048,2048]^T, casts included, median of 3"},
+        "config2_mlp1b_forward": {"value": round(3 * 2 * 32768 * 2048 * 8192 / c2 / 1e12, 4), "unit": "TFLOP/s", "s": round(c2, 2),
+                                  "sample": "Llama-1B-shaped SwiGLU MLP forward, 32768 tokens, one repetition"},
+        "config4_outlier_stress_linear": {"value": round(2 * 2 * TOKENS * DIM * FFN / c4 / 1e12, 4), "unit": "TFLOP/s", "s": round(c4, 2),
+                                          "sample": "4096 -> 11008 linear forward on the outlier-stress activations, row-wise + "
+                                                    "tensor-wise, 16384 tokens, one repetition"},
     }
 
 
