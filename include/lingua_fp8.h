@@ -84,9 +84,13 @@ int l8_cast_rowwise_noalloc(const void *x, int64_t R, int64_t C, int64_t ldx,
  * The amax is used as given (a repeated tensor amax as at :116-118, an amax of an earlier step); where
  * it is smaller than the row's true amax the cast behaves like the ATen one: products up to 464 round
  * to +-448, larger ones give the NaN code.
- *   amax bf16 [R];  q e4m3fn [R,C] (ldq);  scale fp32 [R]
+ *   amax [R], bf16 (amax_dtype = L8_AMAX_BF16: what the reference's amax reductions of bf16 tensors return) or
+ *   fp32 (L8_AMAX_F32: a caller's own fp32 amax, e.g. a history; the reference converts with .float(), so an
+ *   fp32 amax must not be rounded to bf16 on the way);  q e4m3fn [R,C] (ldq);  scale fp32 [R]
  * Requires C % 8 == 0, ldx % 8 == 0, ldq % 8 == 0, 16-byte aligned x / 8-byte aligned q. */
-int l8_cast_rowwise_given_amax(const void *x, int64_t R, int64_t C, int64_t ldx, const void *amax,
+#define L8_AMAX_BF16 0
+#define L8_AMAX_F32 1
+int l8_cast_rowwise_given_amax(const void *x, int64_t R, int64_t C, int64_t ldx, const void *amax, int amax_dtype,
                                void *q, int64_t ldq, float *scale, void *stream);
 
 /* Column amax on its own: col_amax fp32 [C] is overwritten, as above. */
@@ -97,14 +101,14 @@ int l8_col_amax(const void *x, int64_t R, int64_t C, int64_t ldx, float *col_ama
  * amaxes saved by forward). */
 int l8_amax_reduce(const void *amax, int64_t n, void *amax_out, void *stream);
 
-/* Tensor-wise scale -> cast with a device-resident bf16 amax scalar.
+/* Tensor-wise scale -> cast with a device-resident amax scalar (bf16 or fp32, amax_dtype as above).
  * Replaces lingua/float8.py:111 (b_t.t().contiguous()) + :116-118
  * (repeat_interleave of the scalar) + :43-47 (scale()) for the dgrad weight.
  *   transpose == 0 : q is [R,C] (ldq >= C);  != 0 : q is [C,R] (ldq >= R)
  *   scale    fp32 [1]
  * Requires C % 8 == 0, ldx % 8 == 0. */
 int l8_cast_tensorwise(const void *x, int64_t R, int64_t C, int64_t ldx,
-                       const void *amax, int transpose,
+                       const void *amax, int amax_dtype, int transpose,
                        void *q, int64_t ldq, float *scale, void *stream);
 
 /* Column-wise (token-dimension) scale -> cast, written transposed:
@@ -148,6 +152,13 @@ int l8_gemm_nt_ws(const void *A, const void *B, int64_t M, int64_t N, int64_t K,
                   const void *bias, void *C, int64_t ldc, int algo,
                   void *workspace, int64_t workspace_bytes, void *stream);
 int64_t l8_gemm_workspace(void);
+/* A workgroup that owns a shared tile waits for its helpers' partial sums for a bounded time (about a third of a
+ * second; l8_gemm_set_wait_limit).  If the wait runs out -- helpers held up behind other work on the GPU -- the tile
+ * is stored as NaNs (never as a wrong number) and the call still returns L8_OK: the kernel cannot report back.
+ * Every such tile is counted in one 32-bit word of the workspace, at this byte offset; the library never resets it,
+ * so a caller reads it (after synchronising the stream) and compares with what it read before.  No counterpart in
+ * the reference. */
+int64_t l8_gemm_workspace_gave_up_offset(void);
 /* Host arithmetic only: the number of XCDs (0..8) that would share the K range of their last round's tiles out
  * under tile configuration 15, for this problem on a part with `compute_units` compute units (256 on MI355X).
  * 0 = configuration 15 behaves exactly like configuration 12.  No counterpart in the reference. */

@@ -23,14 +23,15 @@ SIGNATURES = {
     "l8_cast_rowwise": [_p, _i64, _i64, _i64, _p, _i64, _p, _p, _p, _p, _i64, _p],
     "l8_cast_rowwise_workspace": [_i64, _i64],
     "l8_cast_rowwise_noalloc": [_p, _i64, _i64, _i64, _p, _i64, _p, _p, _p, _p],
-    "l8_cast_rowwise_given_amax": [_p, _i64, _i64, _i64, _p, _p, _i64, _p, _p],
+    "l8_cast_rowwise_given_amax": [_p, _i64, _i64, _i64, _p, _int, _p, _i64, _p, _p],
     "l8_col_amax": [_p, _i64, _i64, _i64, _p, _p],
     "l8_amax_reduce": [_p, _i64, _p, _p],
-    "l8_cast_tensorwise": [_p, _i64, _i64, _i64, _p, _int, _p, _i64, _p, _p],
+    "l8_cast_tensorwise": [_p, _i64, _i64, _i64, _p, _int, _int, _p, _i64, _p, _p],
     "l8_cast_colwise_transposed": [_p, _i64, _i64, _i64, _p, _p, _i64, _p, _p],
     "l8_gemm_nt": [_p, _p, _i64, _i64, _i64, _i64, _i64, _p, _int, _p, _int, _p, _p, _i64, _int, _p],
     "l8_gemm_nt_ws": [_p, _p, _i64, _i64, _i64, _i64, _i64, _p, _int, _p, _int, _p, _p, _i64, _int, _p, _i64, _p],
     "l8_gemm_workspace": [],
+    "l8_gemm_workspace_gave_up_offset": [],
     "l8_gemm_set_wait_limit": [_int],
     "l8_gemm_shares_k": [_i64, _i64, _i64, _int],
     "l8_swiglu_cast_rowwise": [_p, _p, _i64, _i64, _i64, _i64, _p, _i64, _p, _i64, _p, _p, _p, _p, _i64, _p],
@@ -45,7 +46,7 @@ SIGNATURES = {
     "l8_gemm_algo_name": [_int],
 }
 _RETURNS_STR = {"l8_last_error", "l8_gemm_algo_name"}
-_RETURNS_I64 = {"l8_cast_rowwise_workspace", "l8_gemm_workspace", "l8_swiglu_workspace", "l8_rmsnorm_workspace", "l8_rmsnorm_bwd_workspace"}
+_RETURNS_I64 = {"l8_cast_rowwise_workspace", "l8_gemm_workspace", "l8_gemm_workspace_gave_up_offset", "l8_swiglu_workspace", "l8_rmsnorm_workspace", "l8_rmsnorm_bwd_workspace"}
 
 _lib = None
 _lock = threading.Lock()

@@ -59,9 +59,17 @@ def _run(cmd, verbose):
 def _check_usage(usage) -> None:
     """The persistent GEMM kernel runs at the edge of the register file: a source change that makes the allocator
     spill (or leaves loop state in private memory, which turns every panel load into a loop over lanes) costs a
-    third of its speed and no test would notice.  Such a build fails here instead."""
-    bad = [f"{name}: {u}" for name, u in usage.items()
-           if "gemm_nt_stream_kernel" in name and (u.get("ScratchSize", 0) or u.get("VGPRs Spill", 0))]
+    third of its speed and no test would notice.  Such a build fails here instead -- and so does a build whose
+    compiler remarks could not be read (no entry for the kernel, or an entry without the scratch figure): a check
+    that finds nothing to check must not pass."""
+    stream = {name: u for name, u in usage.items() if "gemm_nt_stream_kernel" in name}
+    if not stream:
+        raise RuntimeError("no register / scratch remarks were parsed for the persistent GEMM kernel "
+                           "(-Rpass-analysis=kernel-resource-usage output missing or in a new format)")
+    unread = [name for name, u in stream.items() if "ScratchSize" not in u or "VGPRs Spill" not in u]
+    if unread:
+        raise RuntimeError("resource remarks without scratch / spill figures for:\n  " + "\n  ".join(unread))
+    bad = [f"{name}: {u}" for name, u in stream.items() if u["ScratchSize"] or u["VGPRs Spill"]]
     if bad:
         raise RuntimeError("the persistent GEMM kernel must not use scratch memory:\n  " + "\n  ".join(bad))
 

@@ -354,14 +354,25 @@ L8_DEV float scale_from_amax_bits32(uint32_t amax_bits) {  // fp32 bit pattern o
   return __uint_as_float(amax_bits == 0x7f800000u ? 0x7f800000u : 0x7fc00000u);
 }
 
+// A device-resident amax scalar, bf16 or fp32 (sign ignored): its scale, and whether it is finite.
+L8_DEV float scale_from_amax_scalar(const void *amax, int amax_f32, bool &finite) {
+  if (amax_f32) {
+    const uint32_t bits = *(const uint32_t *)amax & 0x7fffffffu;
+    finite = bits < 0x7f800000u;
+    return scale_from_amax_bits32(bits);
+  }
+  const uint32_t bits = *(const uint16_t *)amax & 0x7fffu;
+  finite = bits < 0x7f80u;
+  return scale_from_amax_bits16(bits);
+}
+
 __global__ __launch_bounds__(256) void cast_tensorwise_kernel(const uint16_t *__restrict__ x, int64_t R, int C,
-                                                              int64_t ldx, const uint16_t *__restrict__ amax,
+                                                              int64_t ldx, const void *__restrict__ amax, int amax_f32,
                                                               uint8_t *__restrict__ q, int64_t ldq,
                                                               float *__restrict__ scale) {
-  const uint32_t amax_bits = amax[0] & 0x7fffu;
-  const float s = scale_from_amax_bits16(amax_bits);
+  bool finite;
+  const float s = scale_from_amax_scalar(amax, amax_f32, finite);
   const float recip = recip_exact(s);
-  const bool finite = amax_bits < 0x7f80u;
   if (blockIdx.x == 0 && threadIdx.x == 0) scale[0] = s;
   const int cpr = C / 8;  // 16-byte chunks per row
   const int64_t total = R * cpr;
@@ -381,7 +392,7 @@ __global__ __launch_bounds__(256) void cast_tensorwise_kernel(const uint16_t *__
 // product exceeds 448 take the integer conversion, which reproduces the ATen cast there (<= 464 rounds
 // to 448, above gives the NaN code).
 __global__ __launch_bounds__(256) void cast_rowwise_given_amax_kernel(const uint16_t *__restrict__ x, int64_t R, int C,
-                                                                      int64_t ldx, const uint16_t *__restrict__ amax,
+                                                                      int64_t ldx, const void *__restrict__ amax, int amax_f32,
                                                                       uint8_t *__restrict__ q, int64_t ldq,
                                                                       float *__restrict__ scale) {
   const int cpr = C / 8;  // 16-byte chunks per row
@@ -389,7 +400,8 @@ __global__ __launch_bounds__(256) void cast_rowwise_given_amax_kernel(const uint
   for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < total; i += (int64_t)gridDim.x * 256) {
     const int64_t r = i / cpr;
     const int c = (int)(i - r * cpr) * 8;
-    const float s = scale_from_amax(bf16_bits_to_f32(amax[r]));  // clamp(min=EPS) also lifts a negative amax
+    // clamp(min=EPS) also lifts a negative amax
+    const float s = scale_from_amax(amax_f32 ? ((const float *)amax)[r] : bf16_bits_to_f32(((const uint16_t *)amax)[r]));
     const float recip = recip_exact(s);
     if (c == 0) scale[r] = s;
     const v4i v = __builtin_nontemporal_load((const v4i *)(x + r * ldx + c));
@@ -426,7 +438,7 @@ constexpr int kTStride = kTR + 16;           // LDS row stride in bytes
 
 template <bool PER_COL>
 __global__ __launch_bounds__(256) void cast_transposed_kernel(
-    const uint16_t *__restrict__ x, int64_t R, int C, int64_t ldx, const uint16_t *__restrict__ amax_scalar,
+    const uint16_t *__restrict__ x, int64_t R, int C, int64_t ldx, const void *__restrict__ amax_scalar, int amax_f32,
     const uint32_t *__restrict__ col_amax, uint8_t *__restrict__ q, int64_t ldq, float *__restrict__ scale,
     int vec_store) {
   __shared__ __attribute__((aligned(16))) uint8_t tile[kTC * kTStride];
@@ -481,9 +493,7 @@ __global__ __launch_bounds__(256) void cast_transposed_kernel(
 #pragma unroll
     for (int j = 0; j < 8; ++j) rcp[j] = recips[cc * 8 + j];
   } else {
-    const uint32_t amax_bits = amax_scalar[0] & 0x7fffu;
-    const float s = scale_from_amax_bits16(amax_bits);
-    finite = amax_bits < 0x7f80u;
+    const float s = scale_from_amax_scalar(amax_scalar, amax_f32, finite);
     const float rc = recip_exact(s);
 #pragma unroll
     for (int j = 0; j < 8; ++j) rcp[j] = rc;
@@ -724,11 +734,13 @@ extern "C" int l8_cast_rowwise_noalloc(const void *x, int64_t R, int64_t C, int6
   return cast_rowwise_impl("l8_cast_rowwise_noalloc", x, R, C, ldx, q, ldq, scale, amax, col_amax, ws, (hipStream_t)stream);
 }
 
-extern "C" int l8_cast_rowwise_given_amax(const void *x, int64_t R, int64_t C, int64_t ldx, const void *amax, void *q,
-                                          int64_t ldq, float *scale, void *stream) {
+extern "C" int l8_cast_rowwise_given_amax(const void *x, int64_t R, int64_t C, int64_t ldx, const void *amax,
+                                          int amax_dtype, void *q, int64_t ldq, float *scale, void *stream) {
   L8_REQUIRE(R >= 0 && C >= 0, "l8_cast_rowwise_given_amax: negative shape");
   if (R == 0 || C == 0) return L8_OK;
   L8_REQUIRE(x && amax && q && scale, "l8_cast_rowwise_given_amax: null pointer");
+  L8_REQUIRE(amax_dtype == L8_AMAX_BF16 || amax_dtype == L8_AMAX_F32, "l8_cast_rowwise_given_amax: bad amax_dtype %d", amax_dtype);
+  L8_REQUIRE(aligned(amax, amax_dtype == L8_AMAX_F32 ? 4 : 2), "l8_cast_rowwise_given_amax: misaligned amax");
   L8_REQUIRE(C % 8 == 0 && ldx % 8 == 0 && ldx >= C && aligned(x, 16),
              "l8_cast_rowwise_given_amax: C, ldx multiples of 8 and x 16-byte aligned required");
   L8_REQUIRE(ldq >= C && ldq % 8 == 0 && aligned(q, 8),
@@ -739,7 +751,7 @@ extern "C" int l8_cast_rowwise_given_amax(const void *x, int64_t R, int64_t C, i
   const int64_t cap = (int64_t)num_cus() * 16;
   if (blocks > cap) blocks = cap;
   hipLaunchKernelGGL(cast_rowwise_given_amax_kernel, dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream,
-                     (const uint16_t *)x, R, (int)C, ldx, (const uint16_t *)amax, (uint8_t *)q, ldq, scale);
+                     (const uint16_t *)x, R, (int)C, ldx, amax, amax_dtype, (uint8_t *)q, ldq, scale);
   L8_HIP(hipGetLastError());
   return L8_OK;
 }
@@ -775,26 +787,28 @@ extern "C" int l8_amax_reduce(const void *amax, int64_t n, void *amax_out, void 
 }
 
 static int launch_transposed(bool per_col, const void *x, int64_t R, int64_t C, int64_t ldx, const void *amax,
-                             const float *col_amax, void *q, int64_t ldq, float *scale, hipStream_t st) {
+                             int amax_f32, const float *col_amax, void *q, int64_t ldq, float *scale, hipStream_t st) {
   const int64_t gx = ((C + kTC - 1) / kTC) * ((R + kTR - 1) / kTR), gy = 1;
   L8_REQUIRE(gx < (1LL << 31), "transposed cast: shape too large (%lld x %lld)", (long long)R, (long long)C);
   const int vec = (ldq % 16 == 0 && aligned(q, 16)) ? 1 : 0;
   if (per_col)
     hipLaunchKernelGGL((cast_transposed_kernel<true>), dim3((unsigned)gx, (unsigned)gy), dim3(256), 0, st,
-                       (const uint16_t *)x, R, (int)C, ldx, (const uint16_t *)nullptr, (const uint32_t *)col_amax,
+                       (const uint16_t *)x, R, (int)C, ldx, (const void *)nullptr, 0, (const uint32_t *)col_amax,
                        (uint8_t *)q, ldq, scale, vec);
   else
     hipLaunchKernelGGL((cast_transposed_kernel<false>), dim3((unsigned)gx, (unsigned)gy), dim3(256), 0, st,
-                       (const uint16_t *)x, R, (int)C, ldx, (const uint16_t *)amax, (const uint32_t *)nullptr,
+                       (const uint16_t *)x, R, (int)C, ldx, amax, amax_f32, (const uint32_t *)nullptr,
                        (uint8_t *)q, ldq, scale, vec);
   L8_HIP(hipGetLastError());
   return L8_OK;
 }
 
-extern "C" int l8_cast_tensorwise(const void *x, int64_t R, int64_t C, int64_t ldx, const void *amax, int transpose,
-                                  void *q, int64_t ldq, float *scale, void *stream) {
+extern "C" int l8_cast_tensorwise(const void *x, int64_t R, int64_t C, int64_t ldx, const void *amax, int amax_dtype,
+                                  int transpose, void *q, int64_t ldq, float *scale, void *stream) {
   L8_REQUIRE(R >= 0 && C >= 0, "l8_cast_tensorwise: negative shape");
   L8_REQUIRE(amax && scale, "l8_cast_tensorwise: amax and scale must be non-null");
+  L8_REQUIRE(amax_dtype == L8_AMAX_BF16 || amax_dtype == L8_AMAX_F32, "l8_cast_tensorwise: bad amax_dtype %d", amax_dtype);
+  L8_REQUIRE(aligned(amax, amax_dtype == L8_AMAX_F32 ? 4 : 2), "l8_cast_tensorwise: misaligned amax");
   if (R == 0 || C == 0) return L8_OK;
   L8_REQUIRE(x && q, "l8_cast_tensorwise: null pointer");
   L8_REQUIRE(C % 8 == 0 && ldx % 8 == 0 && ldx >= C && aligned(x, 16), "l8_cast_tensorwise: C, ldx multiples of 8 and x 16-byte aligned required");
@@ -802,7 +816,7 @@ extern "C" int l8_cast_tensorwise(const void *x, int64_t R, int64_t C, int64_t l
   hipStream_t st = (hipStream_t)stream;
   if (transpose) {
     L8_REQUIRE(ldq >= R, "l8_cast_tensorwise: transposed output needs ldq >= R");
-    return launch_transposed(false, x, R, C, ldx, amax, nullptr, q, ldq, scale, st);
+    return launch_transposed(false, x, R, C, ldx, amax, amax_dtype, nullptr, q, ldq, scale, st);
   }
   L8_REQUIRE(ldq >= C && ldq % 8 == 0 && aligned(q, 8), "l8_cast_tensorwise: q must be 8-byte aligned with ldq %% 8 == 0, ldq >= C");
   const int64_t total = R * (C / 8);
@@ -810,7 +824,7 @@ extern "C" int l8_cast_tensorwise(const void *x, int64_t R, int64_t C, int64_t l
   const int64_t cap = (int64_t)num_cus() * 16;
   if (blocks > cap) blocks = cap;
   hipLaunchKernelGGL(cast_tensorwise_kernel, dim3((unsigned)blocks), dim3(256), 0, st, (const uint16_t *)x, R, (int)C,
-                     ldx, (const uint16_t *)amax, (uint8_t *)q, ldq, scale);
+                     ldx, amax, amax_dtype, (uint8_t *)q, ldq, scale);
   L8_HIP(hipGetLastError());
   return L8_OK;
 }
@@ -825,5 +839,5 @@ extern "C" int l8_cast_colwise_transposed(const void *x, int64_t R, int64_t C, i
   L8_REQUIRE(C % 8 == 0 && ldx % 8 == 0 && ldx >= C && aligned(x, 16), "l8_cast_colwise_transposed: C, ldx multiples of 8 and x 16-byte aligned required");
   L8_REQUIRE(ldq >= R, "l8_cast_colwise_transposed: ldq >= R required");
   L8_REQUIRE(C < (1LL << 31), "l8_cast_colwise_transposed: C too large");
-  return launch_transposed(true, x, R, C, ldx, nullptr, col_amax, q, ldq, scale, (hipStream_t)stream);
+  return launch_transposed(true, x, R, C, ldx, nullptr, 0, col_amax, q, ldq, scale, (hipStream_t)stream);
 }

@@ -88,7 +88,10 @@ L8_DEV __amdgpu_buffer_rsrc_t make_rsrc(const void *p, uint32_t bytes) {
 // Sharing out the K range of the last, partly filled round of tiles: what a partial tile costs its writer and its
 // reader, in K tiles' time (256 KiB leave a compute unit at ~16 bytes per clock), and the least number of K tiles
 // the split must take off the owners of the tail tiles to be used at all.
-[[maybe_unused]] constexpr int kSkWriteCost = 8, kSkFixCost = 4, kSkMinSaved = 16;  // voffset that is out of range for every resource below
+[[maybe_unused]] constexpr int kSkWriteCost = 8, kSkFixCost = 4, kSkMinSaved = 16;
+// Workspace layout: kSkMaxGrid flag words (one per tail-tile slot), then 64 words of which the first counts the
+// tiles whose owner gave up waiting for a helper (and stored NaNs), then the fp32 tiles of partial sums.
+[[maybe_unused]] constexpr int kSkMaxGridWords = 1024, kSkGaveUpWord = kSkMaxGridWords;
 
 #ifndef L8_GEMM_DIAG
 #define L8_GEMM_DIAG 0
@@ -1071,7 +1074,11 @@ __global__ __launch_bounds__(256) void gemm_nt_stream_kernel(const GemmArgs p) {
         after_store = false;
         if (L8_GEMM_PROF) prof[13] += __builtin_readcyclecounter() - t_b;
       } else {
-        if (!wait_partial(slot)) seg_sa[0] = seg_sa[1] = 0x7fc00000;  // every row scale a NaN
+        if (!wait_partial(slot)) {
+          seg_sa[0] = seg_sa[1] = 0x7fc00000;  // every row scale a NaN
+          // and the host can find out: one more tile poisoned, counted in the workspace (never reset by the library)
+          if (threadIdx.x == 0) atomicAdd(p.sk_flags + kSkGaveUpWord, 1u);
+        }
         if (L8_GEMM_PROF) {
           t_a = __builtin_readcyclecounter();
           prof[14] += t_a - t_b;
@@ -1189,7 +1196,7 @@ static int pick_algo(int64_t M, int64_t N, int64_t K) {
 }
 
 // flags (one 4-byte word per workgroup, first 4 KiB) + one fp32 256x256 tile per workgroup of a persistent launch
-constexpr int64_t kSkMaxGrid = 1024, kSkFlagBytes = kSkMaxGrid * 4, kSkTileBytes = 256 * 256 * 4;
+constexpr int64_t kSkMaxGrid = kSkMaxGridWords, kSkFlagBytes = (kSkMaxGrid + 64) * 4, kSkTileBytes = 256 * 256 * 4;
 static std::atomic<uint32_t> g_sk_epoch{0};
 // polls (about a microsecond each) an owner spends on a helper's flag before it gives up: a third of a second
 static std::atomic<int> g_sk_wait_limit{1 << 18};
@@ -1199,6 +1206,8 @@ extern "C" int l8_gemm_set_wait_limit(int polls) {
   g_sk_wait_limit = polls;
   return L8_OK;
 }
+
+extern "C" int64_t l8_gemm_workspace_gave_up_offset(void) { return (int64_t)kSkGaveUpWord * 4; }
 
 extern "C" int64_t l8_gemm_workspace(void) {
   const int64_t cus8 = (num_cus() / 8) * 8;

@@ -23,9 +23,10 @@ Differences, all deliberate:
   * wgrad is an fp8 product with both operands quantised along the token
     dimension (``config.fp8_wgrad = True``).  Setting it to False restores the
     reference's bf16 ``grad_out.t() @ a`` (lingua/float8.py:123);
-  * the Inductor / CUDA-graph side effects of the converter
-    (lingua/float8.py:162,187-189) have no counterpart: nothing here is traced
-    or compiled at run time;
+  * of the converter's side effects the reset of the dynamo code caches
+    (lingua/float8.py:187) is kept -- modules compiled before the swap trace
+    afresh afterwards -- while the Inductor flag and the CUDA-graph-tree reset
+    (lingua/float8.py:162,189) have no counterpart: no code is generated here;
   * linears applied to the same activation one after the other (w1 / w3, wq /
     wk / wv) share its quantised copy within one forward and one backward
     (``config.share_input_casts``); the reference quantises it once per
@@ -34,6 +35,7 @@ Differences, all deliberate:
     (lingua/float8.py:108) is a no-op for finite gradients and is not issued.
 """
 import re
+import weakref
 from dataclasses import dataclass
 from typing import Callable, Optional
 
@@ -115,8 +117,8 @@ def scale(t: torch.Tensor, amax_t: Optional[torch.Tensor] = None):
             ops.cast_rowwise(t[:, j * cs:(j + 1) * cs], out_q=q[:, j * cs:(j + 1) * cs], out_scale=s[:, j:j + 1])
         return q, s
     if amax_t.shape[0] == t.shape[0] and t.shape[0] != 1:
-        return ops.cast_rowwise_given_amax(t, amax_t.to(torch.bfloat16))
-    return ops.cast_tensorwise(t, amax_t.to(torch.bfloat16), transpose=False)
+        return ops.cast_rowwise_given_amax(t, amax_t)
+    return ops.cast_tensorwise(t, amax_t, transpose=False)
 
 
 def matmul(first, amax_first, second_t, amax_second_t, bias, use_fast_accum: bool = True):
@@ -192,21 +194,32 @@ _fwd_tcast = _LastCast()  # a -> (qat, sat), made in forward when config.save_fp
 
 
 class _WeightCasts:
-    """Quantised copies of weights, one entry per weight storage, valid while pointer, shape, strides, dtype,
-    version counter and stream are what they were (an optimizer step advances the version).  Used only with
-    ``config.cache_weight_casts``."""
+    """Quantised copies of weights, one slot per live weight tensor, valid while pointer, shape, strides, dtype,
+    version counter and stream are what they were (an optimizer step advances the version).  A slot holds the
+    weight by weak reference only and goes away with it, so the cache never holds more than two bytes per
+    parameter of the ``Fp8Linear`` weights that are alive, and a deleted model releases its copies.  Used only
+    with ``config.cache_weight_casts``."""
 
     def __init__(self):
-        self.entries = {}
+        self.entries = {}   # id(weight) -> {"ref": weakref to the weight, "key": ..., "row": ..., "tw": ...}
 
     def _slot(self, w):
         if w.is_inference():
             return None
         key = _LastCast._key(w)
-        slot = self.entries.get(w.data_ptr())
+        slot = self.entries.get(id(w))
+        if slot is not None and slot["ref"]() is not w:
+            slot = None             # the id was handed to another object
         if slot is None or slot["key"] != key:
-            slot = {"key": key, "w": w}
-            self.entries[w.data_ptr()] = slot
+            entries, wid = self.entries, id(w)
+
+            def drop(ref, entries=entries, wid=wid):
+                cur = entries.get(wid)
+                if cur is not None and cur["ref"] is ref:
+                    del entries[wid]
+
+            slot = {"key": key, "ref": weakref.ref(w, drop)}
+            self.entries[wid] = slot
         return slot
 
     def rowwise(self, w):
@@ -424,4 +437,10 @@ def convert_linears_to_fp8(root_module: torch.nn.Module, recipe: str, filter: st
         new_module.bias = module.bias
         return new_module
 
-    return named_replace(replace, root_module)
+    out = named_replace(replace, root_module)
+
+    # As lingua/float8.py:187: a model (or a part of it) compiled before the swap holds graphs traced through the
+    # old nn.Linear modules; dropping the code caches makes the next call trace the converted modules.  The
+    # reference's reset of Inductor's CUDA-graph trees (:189) has no counterpart: nothing here generates code.
+    torch._dynamo.reset_code_caches()
+    return out

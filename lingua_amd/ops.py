@@ -121,19 +121,30 @@ def cast_rowwise(x: torch.Tensor, col_amax: Optional[torch.Tensor] = None, want_
     return q, scale, amax
 
 
+AMAX_BF16, AMAX_F32 = 0, 1
+
+
+def _amax_arg(amax: torch.Tensor, n: int, device, what: str):
+    """An amax handed in by the caller, as the kernels take it: bf16 and fp32 as they are (the reference converts
+    with ``.float()``, lingua/float8.py:44, which is exact for both), any other floating dtype through fp32."""
+    if not amax.is_floating_point() or amax.numel() != n or amax.device != device:
+        raise RuntimeError(f"{what}: amax must be a floating-point tensor with {n} element(s) on the input's device")
+    if amax.dtype not in (torch.bfloat16, torch.float32):
+        amax = amax.float()
+    return amax.contiguous(), (AMAX_F32 if amax.dtype == torch.float32 else AMAX_BF16)
+
+
 def cast_rowwise_given_amax(x: torch.Tensor, amax: torch.Tensor):
-    """scale(x, amax) of lingua/float8.py:43-47 with a row amax [R,1] (bf16) the caller supplies and that is used as
-    given.  Returns (q [R,C] fp8, scale [R,1] fp32)."""
+    """scale(x, amax) of lingua/float8.py:43-47 with a row amax [R,1] (bf16 or fp32) the caller supplies and that is
+    used as given.  Returns (q [R,C] fp8, scale [R,1] fp32)."""
     x = _rows_2d(x, torch.bfloat16, "cast_rowwise_given_amax")
     st = _prep(x, "cast_rowwise_given_amax")
     R, C = x.shape
-    if amax.dtype != torch.bfloat16 or amax.numel() != R or amax.device != x.device:
-        raise RuntimeError("cast_rowwise_given_amax: amax must be bf16 with one element per row, on x's device")
-    amax = amax.contiguous()
+    amax, amax_dtype = _amax_arg(amax, R, x.device, "cast_rowwise_given_amax")
     q = torch.empty((R, C), dtype=torch.float8_e4m3fn, device=x.device)
     scale = torch.empty((R, 1), dtype=torch.float32, device=x.device)
     with _timed("cast_rowwise_given_amax", R * C * 3 + 6 * R, x.device):
-        code = _lib.load().l8_cast_rowwise_given_amax(x.data_ptr(), R, C, _ld(x), amax.data_ptr(), q.data_ptr(), C,
+        code = _lib.load().l8_cast_rowwise_given_amax(x.data_ptr(), R, C, _ld(x), amax.data_ptr(), amax_dtype, q.data_ptr(), C,
                                                       scale.data_ptr(), st)
     _lib.check(code, "l8_cast_rowwise_given_amax")
     return q, scale
@@ -165,17 +176,16 @@ def amax_reduce(amax: torch.Tensor) -> torch.Tensor:
 
 
 def cast_tensorwise(x: torch.Tensor, amax: torch.Tensor, transpose: bool = False):
-    """Tensor-wise scale -> e4m3fn with a device-resident bf16 amax scalar.
+    """Tensor-wise scale -> e4m3fn with a device-resident amax scalar (bf16 or fp32).
     Returns (q [R,C] or [C,R] fp8, scale [1,1] fp32)."""
     x = _rows_2d(x, torch.bfloat16, "cast_tensorwise")
     st = _prep(x, "cast_tensorwise")
-    if amax.dtype != torch.bfloat16 or amax.numel() != 1 or amax.device != x.device:
-        raise RuntimeError("cast_tensorwise: amax must be a one-element bf16 tensor on the same device")
+    amax, amax_dtype = _amax_arg(amax, 1, x.device, "cast_tensorwise")
     R, C = x.shape
     q = torch.empty((C, R) if transpose else (R, C), dtype=torch.float8_e4m3fn, device=x.device)
     scale = torch.empty((1, 1), dtype=torch.float32, device=x.device)
     with _timed("cast_tensorwise_t" if transpose else "cast_tensorwise", R * C * 3 + 4, x.device):
-        code = _lib.load().l8_cast_tensorwise(x.data_ptr(), R, C, _ld(x), amax.data_ptr(), int(transpose),
+        code = _lib.load().l8_cast_tensorwise(x.data_ptr(), R, C, _ld(x), amax.data_ptr(), amax_dtype, int(transpose),
                                               q.data_ptr(), max(q.shape[1], 1), scale.data_ptr(), st)
     _lib.check(code, "l8_cast_tensorwise")
     return q, scale
@@ -198,10 +208,9 @@ def cast_colwise_transposed(x: torch.Tensor, col_amax_f32: torch.Tensor, pad_to:
         q = torch.zeros((C, pad_to), dtype=torch.uint8, device=x.device).view(torch.float8_e4m3fn)
         return q, (torch.clamp(col_amax_f32, min=1e-12) / 448.0).reshape(C, 1)
     Rp = (R + pad_to - 1) // pad_to * pad_to
-    if Rp == R:
-        q = torch.empty((C, R), dtype=torch.float8_e4m3fn, device=x.device)
-    else:
-        q = torch.zeros((C, Rp), dtype=torch.uint8, device=x.device).view(torch.float8_e4m3fn)
+    q = torch.empty((C, Rp), dtype=torch.float8_e4m3fn, device=x.device)
+    if Rp != R:
+        q.view(torch.uint8)[:, R:].zero_()   # the kernel writes columns 0 .. R-1; only the padding is filled here
     scale = torch.empty((C, 1), dtype=torch.float32, device=x.device)
     with _timed("cast_colwise_t", R * C * 3 + 4 * C, x.device):
         code = _lib.load().l8_cast_colwise_transposed(x.data_ptr(), R, C, _ld(x), col_amax_f32.data_ptr(),
@@ -227,6 +236,26 @@ def _gemm_workspace(device: torch.device, stream_ptr, algo: int):
         ws = torch.zeros(_lib.load().l8_gemm_workspace(), dtype=torch.uint8, device=device)
         _gemm_workspaces[key] = ws
     return ws.data_ptr(), ws.numel()
+
+
+def shared_k_tiles_given_up(device=None) -> int:
+    """Number of tiles that tile configuration 15 stored as NaNs since its workspaces on `device` were made,
+    because their owners' bounded wait for a helper's partial sums ran out (the call itself cannot report it).
+    Synchronises the device.  0 is the only healthy answer."""
+    dev = torch.device("cuda", torch.cuda.current_device()) if device is None else torch.device(device)
+    off = _lib.load().l8_gemm_workspace_gave_up_offset()
+    total = 0
+    torch.cuda.synchronize(dev)
+    for (index, _), ws in list(_gemm_workspaces.items()):
+        if index == dev.index:
+            total += int(ws[off:off + 4].view(torch.int32).item())
+    return total
+
+
+def release_gemm_workspaces() -> None:
+    """Frees the workspaces of tile configuration 15 (64 MiB per (device, stream) that used it; otherwise they
+    live as long as the process).  The next call that needs one makes it afresh."""
+    _gemm_workspaces.clear()
 
 
 def gemm_nt(qa: torch.Tensor, qb: torch.Tensor, sa: torch.Tensor, sb: torch.Tensor,

@@ -225,3 +225,35 @@ def test_ffn_hidden_shape_properties_full_size():
     ht = h.t().contiguous()
     q2, s2, _ = ops.cast_rowwise(ht)
     assert torch.equal(qt.view(torch.uint8), q2.view(torch.uint8)) and torch.equal(st, s2)
+
+
+def test_every_finite_amax_lands_on_448_in_the_hardware_converter():
+    """One row (and one column) per finite positive bf16 amax, bit patterns 0x0001 .. 0x7F7F: element 0 is the amax,
+    so `amax * (1 / scale)` -- which may exceed 448 by an ulp or two -- goes through the hardware converter for
+    every amax there is, in the row-wise kernel and in the transposed one (lingua/float8.py:43-47); the other
+    elements are random magnitudes below it."""
+    from lingua_amd import ops
+    n = 0x7F7F
+    g = torch.Generator().manual_seed(77)
+    amax_bits = torch.arange(1, n + 1, dtype=torch.int32)
+    C = 16
+    frac = torch.rand(n, C, generator=g)
+    mag = (frac * (amax_bits.reshape(n, 1) + 1).float()).to(torch.int32).clamp_(max=amax_bits.reshape(n, 1))
+    sign = torch.randint(0, 2, (n, C), generator=g, dtype=torch.int32) << 15
+    bits = mag | sign
+    bits[:, 0] = amax_bits
+    x = bits.to(torch.int16).view(torch.bfloat16)
+    rows = torch.zeros(n + 1, C, dtype=torch.bfloat16)   # + one zero row: a multiple of 8 columns once transposed
+    rows[:n] = x
+    q, s = check_rowwise(rows)
+    above_floor = rows[:n, 0].float() >= 1e-12                       # smaller amaxes are lifted to the floor of the scale
+    assert bool((q.cpu().view(torch.uint8)[:n, 0][above_floor] == 0x7E).all())   # every other amax quantises to +448
+    # the same values with one amax per column, through the transposed kernel
+    xt = rows.t().contiguous()                                       # [16, 32640]
+    xd = dev(xt)
+    col = ops.col_amax(xd)
+    assert bits_equal(col.cpu(), oracle.col_amax(xt).float())
+    qt, st = ops.cast_colwise_transposed(xd, col)
+    qo, so = oracle.cast_colwise_transposed(xt)
+    assert torch.equal(qt.cpu().view(torch.uint8), qo) and bits_equal(st.cpu().reshape(-1), so)
+    assert torch.equal(qt.cpu().view(torch.uint8), q.cpu().view(torch.uint8))  # same bytes either way

@@ -195,6 +195,8 @@ def test_shared_k_range_gives_up_instead_of_hanging():
     qa, qb = fp8(A), fp8(B)
     want = (A @ B.t()).to(torch.bfloat16)
     lib = _lib.load()
+    ops.gemm_nt(qa, qb, one, one, algo=ops.GEMM_ALGO_SHARED_K)   # makes the workspace if this is its first use
+    before = ops.shared_k_tiles_given_up()
     _lib.check(lib.l8_gemm_set_wait_limit(0), "l8_gemm_set_wait_limit")
     try:
         out = ops.gemm_nt(qa, qb, one, one, algo=ops.GEMM_ALGO_SHARED_K)
@@ -202,6 +204,8 @@ def test_shared_k_range_gives_up_instead_of_hanging():
     finally:
         _lib.check(lib.l8_gemm_set_wait_limit(1 << 18), "l8_gemm_set_wait_limit")
     bad = torch.isnan(out)
+    gave_up = ops.shared_k_tiles_given_up() - before
+    assert gave_up == int(bad.reshape(M // 256, 256, N // 256, 256).permute(0, 2, 1, 3).reshape(-1, 256 * 256).any(dim=1).sum())
     assert torch.equal(out[~bad], want[~bad])           # what is not poisoned is right
     if torch.cuda.get_device_properties(0).multi_processor_count == 256:
         tiles = bad.reshape(M // 256, 256, N // 256, 256).permute(0, 2, 1, 3).reshape(-1, 256 * 256)
@@ -209,3 +213,50 @@ def test_shared_k_range_gives_up_instead_of_hanging():
         assert n_bad == int(tiles.any(dim=1).sum())      # whole tiles, nothing partial
         assert n_bad == 8 * 20                           # the 20 tail tiles of each XCD
     assert torch.equal(ops.gemm_nt(qa, qb, one, one, algo=ops.GEMM_ALGO_SHARED_K), want)
+    assert ops.shared_k_tiles_given_up() - before == gave_up      # the healthy call adds nothing
+
+
+# The persistent kernel with a bias, on problems where a workgroup computes several tiles (scales and bias are
+# requested afresh per tile while the stores of the tile before are still in flight): ragged edges in both
+# directions, a K tail, 17 x 18 and 33 x 34 tiles.
+SHAPES_BIAS_PERSISTENT = [(4100, 4360, 1040), (8200, 8456, 1040)]
+
+
+@pytest.mark.parametrize("algo", [0, 12])
+@pytest.mark.parametrize("mnk", SHAPES_BIAS_PERSISTENT)
+def test_persistent_kernel_with_bias_exact_integer_operands(algo, mnk):
+    from lingua_amd import ops
+    M, N, K = mnk
+    g = torch.Generator(device="cuda").manual_seed(M + algo)
+    A = torch.randint(-1, 2, (M, K), generator=g, device="cuda").float()
+    B = torch.randint(-1, 2, (N, K), generator=g, device="cuda").float()
+    sa = torch.tensor([2.0 ** (i % 5 - 2) for i in range(M)], device="cuda").reshape(M, 1)
+    sb = torch.tensor([2.0 ** (i % 3) for i in range(N)], device="cuda").reshape(N, 1)
+    bias = torch.randint(-64, 65, (N,), generator=g, device="cuda").to(torch.bfloat16)  # integers: exact sums
+    torch.backends.cuda.matmul.allow_tf32 = False
+    prod = A @ B.t()  # integer sums below 2^24: exact in fp32
+    for sa_, sb_ in ((sa, sb), (sa[:1], sb[:1]), (sa, sb[:1])):
+        out = ops.gemm_nt(fp8(A), fp8(B), sa_, sb_, bias, algo=algo)
+        want = (prod * sa_ * sb_.t() + bias.float()).to(torch.bfloat16)
+        assert torch.equal(out, want), (algo, mnk, sa_.numel(), sb_.numel())
+        # and the same bits as the plain one-workgroup-per-tile kernel
+        assert torch.equal(out, ops.gemm_nt(fp8(A), fp8(B), sa_, sb_, bias, algo=5))
+
+
+@pytest.mark.parametrize("algo", [0, 12])
+def test_persistent_kernel_with_bias_random_operands_vs_oracle_rows(algo):
+    from lingua_amd import ops
+    for (M, N, K) in SHAPES_BIAS_PERSISTENT + [(16384, 4096, 4096)]:
+        g = torch.Generator().manual_seed(M + N)
+        qa, qb = random_fp8_bytes((M, K), g), random_fp8_bytes((N, K), g)
+        sa = torch.rand(M, 1, generator=g) + 0.5
+        sb = torch.rand(N, 1, generator=g) + 0.5
+        bias = (torch.randn(N, generator=g) * 5e4).to(torch.bfloat16)   # the size of the products: it must show
+        A, B = qa.cuda().view(torch.float8_e4m3fn), qb.cuda().view(torch.float8_e4m3fn)
+        rows = torch.cat([torch.arange(0, M, max(1, M // 40))[:40], torch.arange(M - 6, M)])
+        for sa_, sb_ in ((sa, sb), (sa[:1], sb[:1])):
+            out = ops.gemm_nt(A, B, sa_.cuda(), sb_.cuda(), bias.cuda(), algo=algo)
+            want = oracle.gemm_nt(qa[rows], qb, sa_[rows] if sa_.numel() == M else sa_, sb_, bias)
+            assert rel_l2(out[rows.cuda()], want) <= TOL, (algo, M, N, K)
+            plain = ops.gemm_nt(A, B, sa_.cuda(), sb_.cuda(), bias.cuda(), algo=5)
+            assert rel_l2(out, plain) <= 1e-4, (algo, M, N, K)  # the whole matrix, against the plain kernel

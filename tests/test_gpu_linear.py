@@ -605,3 +605,62 @@ def test_weight_casts_kept_between_optimizer_steps():
     assert again_plain == 2 and again_cached == 2  # a changed weight is quantised again
     for a, b in zip(plain, cached):
         assert torch.equal(a.view(torch.int16), b.view(torch.int16))
+
+
+def test_large_linear_with_bias_vs_oracle():
+    """nn.Linear(4096, 4096, bias=True) on 4096 tokens: 256 tiles, so forward takes the persistent kernel's bias
+    instantiation; forward (lingua/float8.py:65-73 with the bias fused), dgrad and fp8 wgrad against the oracle on
+    row samples, grad_bias against the oracle's column sum (lingua/float8.py:127)."""
+    from lingua_amd import Fp8Linear
+    M, K, N = 4096, 4096, 4096
+    lin = Fp8Linear(K, N, bias=True, device="cuda", dtype=torch.bfloat16)
+    w = seeded_bf16((N, K), 0.02, seed=51)
+    b = seeded_bf16((N,), 2.0, seed=52)
+    with torch.no_grad():
+        lin.weight.copy_(w)
+        lin.bias.copy_(b)
+    x = seeded_bf16((M, K), 1.0, seed=53)
+    go = seeded_bf16((M, N), 1e-2, seed=54)
+    xd = x.cuda().requires_grad_(True)
+    y = lin(xd)
+    y.backward(go.cuda())
+    rows = torch.arange(0, M, M // 32)[:32]
+    qx, sx, _ = oracle.cast_rowwise(x[rows])
+    qw, sw, _ = oracle.cast_rowwise(w)
+    assert rel_l2(y[rows.cuda()], oracle.gemm_nt(qx, qw, sx, sw, b)) <= TOL
+    assert rel_l2(xd.grad[rows.cuda()], oracle.linear_dgrad(go[rows], w)) <= TOL
+    # wgrad reduces over all tokens: a sample of output rows (columns of grad_out) against the oracle
+    cols = torch.arange(0, N, N // 24)[:24]
+    assert rel_l2(lin.weight.grad[cols.cuda()], oracle.linear_wgrad_fp8(go[:, cols].contiguous(), x)) <= TOL
+    assert rel_l2(lin.bias.grad, oracle.col_sum(go)) <= 5e-3
+
+
+def test_weight_cast_cache_lets_go_of_a_deleted_model():
+    """config.cache_weight_casts holds each weight by weak reference: deleting the model frees the weights and
+    their quantised copies (device memory returns to where it was), and the cache has no slot left."""
+    import gc
+    from lingua_amd import Fp8Linear, float8
+    float8.clear_cast_memos()
+    gc.collect()
+    torch.cuda.synchronize()
+    base = torch.cuda.memory_allocated()
+    old = float8.config.cache_weight_casts
+    float8.config.cache_weight_casts = True
+    try:
+        model = torch.nn.Sequential(*[Fp8Linear(512, 512, bias=False, device="cuda", dtype=torch.bfloat16) for _ in range(4)])
+        x = seeded_bf16((64, 512), seed=3).cuda().requires_grad_(True)
+        for _ in range(2):
+            model(x).sum().backward()
+        assert len(float8._weight_casts.entries) == 4
+        held = torch.cuda.memory_allocated() - base
+        assert held >= 4 * 512 * 512 * 4          # bf16 weights + two one-byte copies each
+        del model
+        x.grad = None
+        del x
+        float8._fwd_cast.clear(); float8._bwd_cast.clear(); float8._fwd_tcast.clear()   # the activation memos only
+        gc.collect()
+        assert len(float8._weight_casts.entries) == 0
+        assert torch.cuda.memory_allocated() == base
+    finally:
+        float8.config.cache_weight_casts = old
+        float8.clear_cast_memos()

@@ -96,7 +96,7 @@ def test_cast_transposed_sweep():
                 ld = (ld + 7) // 8 * 8
             q = torch.full((rows, ld), FILL, dtype=torch.uint8, device="cuda")
             s1 = torch.empty(1, dtype=torch.float32, device="cuda")
-            L.check(lib.l8_cast_tensorwise(x.data_ptr(), R, C, ldx, amax.cuda().data_ptr(), transpose, q.data_ptr(), ld,
+            L.check(lib.l8_cast_tensorwise(x.data_ptr(), R, C, ldx, amax.cuda().data_ptr(), 0, transpose, q.data_ptr(), ld,
                                            s1.data_ptr(), _stream()), "l8_cast_tensorwise")
             wq, wsc = oracle.cast_tensorwise(xc, amax, transpose=bool(transpose))
             assert torch.equal(q.cpu()[:, :cols], wq), tag + (transpose,)

@@ -105,6 +105,21 @@ def test_scale_uses_the_row_amax_it_is_given():
     q4, s4 = f8.scale(xd, bad.cuda())
     want_q, want_s = rt.scale(x, bad)
     assert fp8_equal_mod_nan_sign(q4, want_q) and bits_equal(s4.cpu(), want_s)
+    # (5) an fp32 amax that is not a bf16 value (a history of amaxes, a margin): the reference converts with
+    # .float() (lingua/float8.py:44), so no bit of it may be lost; row-wise and tensor-wise
+    amax32 = true_amax.float() * 1.003 + 1e-3
+    assert not torch.equal(amax32.to(torch.bfloat16).float(), amax32)
+    q5, s5 = f8.scale(xd, amax32.cuda())
+    want_q, want_s = rt.scale(x, amax32)
+    assert torch.equal(q5.cpu().view(torch.uint8), want_q.view(torch.uint8)) and bits_equal(s5.cpu(), want_s)
+    t32 = (amax32.amax() * 1.01).reshape(1, 1)
+    q6, s6 = f8.scale(xd, t32.cuda())
+    want_q, want_s = rt.scale(x, t32)
+    assert torch.equal(q6.cpu().view(torch.uint8), want_q.view(torch.uint8)) and bits_equal(s6.cpu().reshape(-1), want_s.reshape(-1))
+    # fp16 goes through fp32, exactly as .float() would take it
+    q7, s7 = f8.scale(xd, amax32.half().cuda())
+    want_q, want_s = rt.scale(x, amax32.half())
+    assert torch.equal(q7.cpu().view(torch.uint8), want_q.view(torch.uint8)) and bits_equal(s7.cpu(), want_s)
 
 
 def test_matmul_called_as_the_reference_dgrad_calls_it():

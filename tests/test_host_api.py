@@ -40,7 +40,7 @@ def test_argument_validation_happens_before_launch():
     assert lib.l8_gemm_nt(fake + 1, fake, 4, 4, 16, 16, 16, fake, 1, fake, 1, None, fake, 4, 0, None) == -1
     assert lib.l8_cast_rowwise(fake, 4, 12, 12, fake, 12, fake, None, None, None, 0, None) == -1
     assert lib.l8_cast_rowwise(fake, -1, 8, 8, fake, 8, fake, None, None, None, 0, None) == -1
-    assert lib.l8_cast_tensorwise(fake, 4, 8, 8, None, 0, fake, 8, fake, None) == -1
+    assert lib.l8_cast_tensorwise(fake, 4, 8, 8, None, 0, 0, fake, 8, fake, None) == -1
     assert lib.l8_cast_colwise_transposed(fake, 4, 8, 8, None, fake, 4, fake, None) == -1
     # empty problems are accepted and do nothing
     assert lib.l8_cast_rowwise(None, 0, 8, 8, None, 8, None, None, None, None, 0, None) == 0
@@ -224,3 +224,39 @@ def test_build_refuses_a_persistent_gemm_kernel_that_uses_scratch():
         bad["_ZN2l821gemm_nt_stream_kernelILi4ELb0ELb0EEEvNS_8GemmArgsE"][field] = 12
         with pytest.raises(RuntimeError):
             build._check_usage(bad)
+    # a check that finds nothing to check must fail too: no remark parsed at all, or one without the figures
+    with pytest.raises(RuntimeError):
+        build._check_usage({})
+    with pytest.raises(RuntimeError):
+        build._check_usage({"_ZN2l821gemm_nt_stream_kernelILi4ELb0ELb0EEEvNS_8GemmArgsE": {"VGPRs": 158, "AGPRs": 256}})
+    # and the shipped build's record lists every instantiation of the persistent kernel
+    usage_file = os.path.join(os.path.dirname(build.LIB_PATH), "build", "resource_usage.txt")
+    if os.path.exists(usage_file):
+        text = open(usage_file).read()
+        for inst in ("ILi4ELb0ELb0E", "ILi4ELb1ELb0E", "ILi4ELb0ELb1E", "ILi8ELb0ELb0E", "ILi2ELb0ELb0E", "ILi16ELb0ELb0E"):
+            assert "gemm_nt_stream_kernel" + inst in text, inst
+
+
+def test_converter_drops_compiled_code_like_the_reference():
+    """lingua/float8.py:187 resets the dynamo code caches after the swap ("force re-compile everything"): a
+    module compiled before the conversion is traced again by its next call.  Runs on the CPU with a filter that
+    matches nothing, so no Fp8Linear (GPU only) is executed."""
+    import torch
+    from lingua_amd import convert_linears_to_fp8
+    traces = []
+
+    def backend(gm, example_inputs):
+        traces.append(len(traces))
+        return gm.forward
+
+    torch._dynamo.reset()
+    model = torch.nn.Sequential(torch.nn.Linear(8, 8), torch.nn.ReLU())
+    compiled = torch.compile(model, backend=backend)
+    x = torch.randn(2, 8)
+    compiled(x)
+    compiled(x)
+    assert len(traces) == 1                    # second call served from the code cache
+    assert convert_linears_to_fp8(model, "rowwise", r"layers\.[0-9]+\.") is model
+    compiled(x)
+    assert len(traces) == 2                    # traced afresh after the conversion
+    torch._dynamo.reset()
