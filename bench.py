@@ -30,12 +30,24 @@ DIM, FFN, TOKENS = 4096, 11008, 16384
 STEP_FLOP = 18 * TOKENS * DIM * FFN          # 9 GEMMs x 2*M*N*K
 PEAK_FP8_TFLOPS = 5000.0                     # MI355X dense fp8 MFMA, published
 PEAK_HBM_GBPS = 8000.0                       # MI355X HBM3E, published
-# HBM-side bytes per GEMM launch from rocprofv3 FETCH_SIZE / WRITE_SIZE, each scaled by what the same counter reads
-# for a 256 MiB copy (profiles/gemm_nt_7b_hbm_traffic.txt), mean over the three products the step launches three
-# times each: forward 1.527 GB, dgrad 1.234 GB, wgrad 1.435 GB (algorithmic: 473 / 360 / 338 MB).  A counter run
-# cannot share a process with the timed steps (it slows the kernels by ~8 %), so the figure is carried over from
-# the profile of this same kernel and shapes and named as such in the JSON line.
-GEMM_TRAFFIC_BYTES = 1_370_000_000
+# HBM-side bytes per GEMM launch come from rocprofv3 FETCH_SIZE / WRITE_SIZE runs, each scaled by what the same
+# counter reads for a 256 MiB copy, mean over the three products the step launches three times each.  A counter run
+# cannot share a process with the timed steps (it slows the kernels by ~8 %), so the figure is read from the
+# committed summary of those runs (one line "roofline.traffic bytes per launch: N") and named as such in the line.
+TRAFFIC_PROFILE = os.path.join(ROOT, "profiles", "gemm_nt_7b_hbm_traffic.txt")
+
+
+def gemm_traffic_bytes():
+    """The `roofline.traffic` figure and the kernel it was measured on, from the committed counter summary; a
+    missing or unreadable summary is an error, not a silent constant."""
+    import re
+    with open(TRAFFIC_PROFILE) as f:
+        text = f.read()
+    m = re.search(r"^roofline\.traffic bytes per launch: (\d+)\s*$", text, re.M)
+    k = re.search(r"^kernel: (\S+)\s*$", text, re.M)
+    if not m or not k:
+        raise RuntimeError(f"{TRAFFIC_PROFILE} holds no 'roofline.traffic bytes per launch:' / 'kernel:' line")
+    return int(m.group(1)), k.group(1)
 
 
 def parse():
@@ -126,7 +138,7 @@ def cpu_baseline(torch, sample_tokens):
     c2 = time.perf_counter() - t0
     del x2, v1, v2, v3
     # configs[3]: the 4096 -> 11008 linear on the outlier-stress activations, row-wise and tensor-wise, one repetition
-    from workloads import outlier_stress_input, seeded_bf16
+    from bench_workloads import outlier_stress_input, seeded_bf16
     x4, _, _ = outlier_stress_input(rows=TOKENS, cols=DIM, seed=0)
     w4 = seeded_bf16((FFN, DIM), 0.02, seed=1)
     t0 = time.perf_counter()
@@ -151,6 +163,125 @@ def cpu_baseline(torch, sample_tokens):
     }
 
 
+def kernel_table(records):
+    """{kernel: launches, avg_ms, and TFLOP/s (GEMM) or GB/s + fraction of HBM peak (everything else)} from the
+    (name, start event, end event, algorithmic work) records of lingua_amd.ops.kernel_timer."""
+    agg = {}
+    for name, e0, e1, work in records:
+        a = agg.setdefault(name, [0, 0.0, 0])
+        a[0] += 1
+        a[1] += e0.elapsed_time(e1)
+        a[2] += work
+    table = {}
+    for name, (n, ms, work) in agg.items():
+        if name == "gemm_nt":
+            table[name] = {"launches": n, "avg_ms": round(ms / n, 4), "TFLOP/s": round(work / (ms * 1e-3) / 1e12, 1)}
+        else:
+            gbps = work / (ms * 1e-3) / 1e9
+            table[name] = {"launches": n, "avg_ms": round(ms / n, 4), "GB/s": round(gbps, 1),
+                           "frac_hbm": round(gbps / PEAK_HBM_GBPS, 4)}
+    return table
+
+
+def gemm_shape_table(torch, dev, iters=20, warm=5):
+    """The GEMM alone on the products of the Llama-1B-shaped linears (dim 2048, ffn 8192, 16384 tokens:
+    lingua/transformer.py:357-359,406,469-471 at that size; wq/wk/wv also as one fused product), of configs[0]
+    and configs[1], and on the three 7B products: ms, TFLOP/s, fraction of the fp8 peak and the tile
+    configuration the library picks, operands quantised from seeded normal data."""
+    from lingua_amd import ops
+    shapes = [("1B wq/wk/wv/wo fwd and dgrad", 16384, 2048, 2048), ("1B wq+wk+wv as one product, fwd", 16384, 6144, 2048),
+              ("1B w1/w3 fwd, w2 dgrad", 16384, 8192, 2048), ("1B w2 fwd, w1/w3 dgrad", 16384, 2048, 8192),
+              ("1B wq/wk/wv/wo wgrad", 2048, 2048, 16384), ("1B w1/w3 wgrad", 8192, 2048, 16384),
+              ("1B w2 wgrad", 2048, 8192, 16384), ("config 1 linear fwd", 4096, 2048, 2048),
+              ("config 2 w1/w3 fwd", 32768, 8192, 2048), ("config 2 w2 fwd", 32768, 2048, 8192),
+              ("7B fwd", TOKENS, FFN, DIM), ("7B dgrad", TOKENS, DIM, FFN), ("7B wgrad", FFN, DIM, TOKENS)]
+    g = torch.Generator(device=dev).manual_seed(11)
+    rows = []
+    for what, M, N, K in shapes:
+        a = torch.randn(M, K, generator=g, device=dev).to(torch.bfloat16)
+        b = (torch.randn(N, K, generator=g, device=dev) * 0.02).to(torch.bfloat16)
+        qa, sa, _ = ops.cast_rowwise(a)
+        qb, sb, _ = ops.cast_rowwise(b)
+        out = torch.empty(M, N, dtype=torch.bfloat16, device=dev)
+        for _ in range(warm):
+            ops.gemm_nt(qa, qb, sa, sb, out=out)
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(iters):
+            ops.gemm_nt(qa, qb, sa, sb, out=out)
+        e1.record()
+        torch.cuda.synchronize()
+        ms = e0.elapsed_time(e1) / iters
+        tf = 2 * M * N * K / (ms * 1e-3) / 1e12
+        rows.append({"what": what, "M": M, "N": N, "K": K, "ms": round(ms, 4), "TFLOP/s": round(tf, 1),
+                     "frac_of_fp8_peak": round(tf / PEAK_FP8_TFLOPS, 4), "kernel": ops.gemm_pick(M, N, K)[1]})
+        del a, b, qa, qb, out
+    return rows
+
+
+def config_figures(torch, dev, iters=20, warm=5):
+    """GPU figures for the configurations the CPU baseline also times: configs[0] (one row-wise linear forward,
+    x [4096,2048], W [2048,2048], casts included), configs[1] (Llama-1B-shaped SwiGLU MLP forward, 32768 tokens,
+    through convert_linears_to_fp8) and the configs[3] linear (4096 -> 11008 forward on 16384 outlier-stress
+    tokens, row-wise and tensor-wise: casts + GEMM each)."""
+    from torch import nn
+    from lingua_amd import Fp8Linear, convert_linears_to_fp8, ops
+    from bench_workloads import outlier_stress_input, seeded_bf16
+
+    def clock(fn):
+        for _ in range(warm):
+            fn()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(iters):
+            fn()
+        e1.record()
+        torch.cuda.synchronize()
+        return e0.elapsed_time(e1) / iters
+
+    res = {}
+    with torch.no_grad():
+        lin = Fp8Linear(2048, 2048, bias=False, device=dev, dtype=torch.bfloat16)
+        lin.weight.copy_(seeded_bf16((2048, 2048), 0.02, seed=1).to(dev))
+        x1 = seeded_bf16((4096, 2048), 1.0, seed=0).to(dev)
+        ms = clock(lambda: lin(x1))
+        res["config1_linear_forward"] = {"ms": round(ms, 4), "TFLOP/s": round(2 * 4096 * 2048 * 2048 / (ms * 1e-3) / 1e12, 1),
+                                         "what": "x [4096,2048] @ W [2048,2048]^T, both casts + GEMM per call"}
+        mlp = make_mlp(torch, nn, 2048, 8192, dev)
+        mlp = convert_linears_to_fp8(nn.ModuleDict({"layers": nn.ModuleList([mlp])}), "rowwise", r"layers\.[0-9]+\.")["layers"][0]
+        x2 = seeded_bf16((32768, 2048), 1.0, seed=2).to(dev)
+        ms = clock(lambda: mlp(x2))
+        flop2 = 3 * 2 * 32768 * 2048 * 8192
+        res["config2_mlp1b_forward"] = {"ms": round(ms, 4), "TFLOP/s": round(flop2 / (ms * 1e-3) / 1e12, 1),
+                                        "frac_of_fp8_peak": round(flop2 / (ms * 1e-3) / 1e12 / PEAK_FP8_TFLOPS, 4),
+                                        "what": "Llama-1B-shaped SwiGLU MLP forward, 32768 tokens: 3 GEMMs, 5 casts, silu and mul in bf16"}
+        del mlp, x2, lin, x1
+        torch.cuda.empty_cache()
+        x4, _, _ = outlier_stress_input(rows=TOKENS, cols=DIM, seed=0)
+        x4 = x4.to(dev)
+        w4 = seeded_bf16((FFN, DIM), 0.02, seed=1).to(dev)
+
+        def rowwise():
+            qx, sx, _ = ops.cast_rowwise(x4)
+            qw, sw, _ = ops.cast_rowwise(w4)
+            return ops.gemm_nt(qx, qw, sx, sw)
+
+        def tensorwise():
+            _, _, ax = ops.cast_rowwise(x4, want_q=False)
+            _, _, aw = ops.cast_rowwise(w4, want_q=False)
+            qx, sx = ops.cast_tensorwise(x4, ops.amax_reduce(ax))
+            qw, sw = ops.cast_tensorwise(w4, ops.amax_reduce(aw))
+            return ops.gemm_nt(qx, qw, sx, sw)
+
+        flop4 = 2 * TOKENS * DIM * FFN
+        for name, fn in (("rowwise", rowwise), ("tensorwise", tensorwise)):
+            ms = clock(fn)
+            res["config4_linear_forward_" + name] = {"ms": round(ms, 4), "TFLOP/s": round(flop4 / (ms * 1e-3) / 1e12, 1),
+                                                     "what": "4096 -> 11008 linear forward on 16384 outlier-stress tokens, "
+                                                             + name + " scaling of both operands, amax + casts + GEMM per call"}
+    return res
+
+
 def extras(torch, mlp, timed, args):
     """Side measurements, never part of `value`:
     fused_swiglu     the same MLP, same recipe, through lingua_amd.swiglu.Fp8FeedForward (gate fused into the casts,
@@ -163,6 +294,11 @@ def extras(torch, mlp, timed, args):
     dt = timed(fused, None)
     res["fused_swiglu"] = {"value": round(STEP_FLOP / (dt / args.steps) / 1e12, 2), "unit": "TFLOP/s",
                            "ms_per_step": round(dt / args.steps * 1e3, 4)}
+    if not args.no_kernel_timing:
+        # the fused gate kernels' own rates: a second pass with every launch bracketed (not part of the figure above)
+        rec = []
+        timed(fused, rec, {"swiglu_cast_rowwise", "swiglu_bwd_cast_rowwise"})
+        res["fused_swiglu"]["kernels"] = kernel_table(rec)
     try:
         dev = mlp.w1.weight.device
         total_ms = 0.0
@@ -194,7 +330,11 @@ def more_extras(torch, dev, args):
     res = {}
     res["linear7b"] = measure_linear7b(args, torch, dev)
     torch.cuda.empty_cache()
-    from workloads import outlier_stress_figures
+    res["gemm_shapes"] = gemm_shape_table(torch, dev)
+    torch.cuda.empty_cache()
+    res.update(config_figures(torch, dev))
+    torch.cuda.empty_cache()
+    from bench_workloads import outlier_stress_figures
     fig, tensors = outlier_stress_figures(TOKENS)
     del tensors
     torch.cuda.empty_cache()
@@ -254,7 +394,7 @@ def run_linear7b(args, torch, dev):
 def measure_llama1b(torch, dev, steps, warmup, fused_too=True):
     """configs[4]: tokens/s of a Llama-1B-shaped forward+backward step, block linears in row-wise fp8."""
     from lingua_amd import convert_linears_to_fp8
-    from workloads import Llama, LLAMA_1B, llama_flops_per_token
+    from bench_workloads import Llama, LLAMA_1B, llama_flops_per_token
     B, S = 4, 4096
     with torch.device(dev):
         model = Llama(**LLAMA_1B).to(torch.bfloat16)
@@ -283,6 +423,31 @@ def measure_llama1b(torch, dev, steps, warmup, fused_too=True):
         return (time.perf_counter() - t0) / steps
 
     dt = timed(model)
+
+    def kernel_share(m, step_dt):
+        """Two more steps with every launch of this library bracketed by events: the share of the step's time that
+        its kernels account for (the rest is the stand-in model's plain PyTorch: attention, rope, embeddings, loss,
+        residual adds, and the bf16 output head), and the kernels' own table."""
+        from lingua_amd import ops
+        params = list(m.parameters())
+        rec = []
+        ops.kernel_timer, ops.kernel_timer_names = rec, None
+        try:
+            for _ in range(2):
+                for p in params:
+                    p.grad = None
+                bump_versions(torch, params)
+                m(tokens, labels).backward()
+            torch.cuda.synchronize()
+        finally:
+            ops.kernel_timer, ops.kernel_timer_names = None, None
+        table = kernel_table(rec)
+        ms = sum(e0.elapsed_time(e1) for _, e0, e1, _ in rec) / 2
+        gemm_ms = sum(e0.elapsed_time(e1) for name, e0, e1, _ in rec if name == "gemm_nt") / 2
+        return {"fp8_kernels_ms_per_step": round(ms, 3), "fp8_gemm_ms_per_step": round(gemm_ms, 3),
+                "share_of_step": round(ms / (step_dt * 1e3), 4), "kernels": table}
+
+    share = kernel_share(model, dt)
     fused_dt = None
     if fused_too:
         # same weights, gate fused into the casts, norms that hand their output over quantised, one product for wq/wk/wv
@@ -296,6 +461,7 @@ def measure_llama1b(torch, dev, steps, warmup, fused_too=True):
            "model_TFLOP/s": round(fpt * B * S / dt / 1e12, 1), "fp8_linear_TFLOP/s_if_alone": round(fp8_flop / dt / 1e12, 1),
            "what": "Llama-1B-shaped step fwd+bwd (configs[4]): 25 layers, dim 2048, ffn 8192, vocab 128256, 4 x 4096 tokens; "
                    "block linears through convert_linears_to_fp8, the rest of the step is the stand-in model's plain PyTorch"}
+    res["fp8_path"] = share
     if fused_dt is not None:
         res["fused_swiglu_and_rmsnorm"] = {"value": round(B * S / fused_dt, 1), "unit": "tokens/s",
                                            "ms_per_step": round(fused_dt * 1e3, 3)}
@@ -305,7 +471,7 @@ def measure_llama1b(torch, dev, steps, warmup, fused_too=True):
 
 
 def run_llama1b(args, torch, dev):
-    from workloads import LLAMA_1B
+    from bench_workloads import LLAMA_1B
     r = measure_llama1b(torch, dev, args.steps, args.warmup, fused_too=not args.no_extras)
     print(json.dumps({
         "metric": "Llama-1B forward+backward tokens/s, block linears fp8 row-wise", "value": r["value"],
@@ -314,6 +480,7 @@ def run_llama1b(args, torch, dev):
         "config": {"workload": "llama-1B step fwd+bwd (configs[4])", "batch": 4, "seq_len": 4096, **LLAMA_1B},
         "model_TFLOP/s": r["model_TFLOP/s"],
         "fp8_linear_TFLOP/s_if_alone": r["fp8_linear_TFLOP/s_if_alone"],
+        "fp8_path": r["fp8_path"],
         "extras": {"fused_swiglu_and_rmsnorm": r.get("fused_swiglu_and_rmsnorm")},
     }))
 
@@ -465,27 +632,28 @@ def main():
     roofline = None
     kernels = {}
     if records:
+        kernels = kernel_table(records)
         agg = {}
         for name, e0, e1, work in records:
-            ms = e0.elapsed_time(e1)
             a = agg.setdefault(name, [0, 0.0, 0])
             a[0] += 1
-            a[1] += ms
+            a[1] += e0.elapsed_time(e1)
             a[2] += work
-        for name, (n, ms, work) in agg.items():
-            if name == "gemm_nt":
-                kernels[name] = {"launches": n, "avg_ms": round(ms / n, 4), "TFLOP/s": round(work / (ms * 1e-3) / 1e12, 1)}
-            else:
-                gbps = work / (ms * 1e-3) / 1e9
-                kernels[name] = {"launches": n, "avg_ms": round(ms / n, 4), "GB/s": round(gbps, 1),
-                                 "frac_hbm": round(gbps / PEAK_HBM_GBPS, 4)}
         n, ms, work = agg["gemm_nt"]
         achieved = work / (ms * 1e-3) / 1e12
-        roofline = {"kernel": "gemm_nt_stream_kernel<4,false,false> (fp8 e4m3 NT GEMM, 2*16384*4096*11008 flop per launch; forward, dgrad and wgrad products)",
+        picked = {ops.gemm_pick(*mnk) for mnk in ((TOKENS, FFN, DIM), (TOKENS, DIM, FFN), (FFN, DIM, TOKENS))}
+        if args.algo:
+            picked = {(args.algo, ops.gemm_algos()[args.algo - 1])}
+        traffic, traffic_kernel = gemm_traffic_bytes()
+        names = sorted(name for _, name in picked)
+        roofline = {"kernel": " / ".join(names) + " (fp8 e4m3 NT GEMM, 2*16384*4096*11008 flop per launch; forward, dgrad and wgrad products)",
                     "bound": "mfma", "achieved": round(achieved, 1), "peak": PEAK_FP8_TFLOPS, "unit": "TFLOP/s",
-                    "frac": round(achieved / PEAK_FP8_TFLOPS, 4), "traffic": GEMM_TRAFFIC_BYTES,
+                    "frac": round(achieved / PEAK_FP8_TFLOPS, 4),
+                    # counters of another tile configuration say nothing about this one
+                    "traffic": traffic if names == [traffic_kernel] else None,
                     "traffic_unit": "bytes per launch, mean of the step's three products (algorithmic: 390 MB); from "
-                                    "profiles/gemm_nt_7b_hbm_traffic.txt (rocprofv3 FETCH_SIZE / WRITE_SIZE runs of this kernel)"}
+                                    "profiles/gemm_nt_7b_hbm_traffic.txt (rocprofv3 FETCH_SIZE / WRITE_SIZE runs of "
+                                    + traffic_kernel + ")"}
 
     out = {
         "metric": "fp8 rowwise linear fwd+bwd TFLOP/s at 7B MLP",

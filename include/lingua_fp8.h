@@ -229,6 +229,10 @@ int64_t l8_rmsnorm_bwd_workspace(int64_t R, int64_t C);
 int l8_gemm_algo_count(void);
 /* human-readable description of tile configuration `algo` (1-based), or NULL */
 const char *l8_gemm_algo_name(int algo);
+/* Host arithmetic only: the tile configuration that `algo = 0` resolves to for an M x N x K problem on the
+ * current device when the operands allow every kernel (aligned, N % 8 == 0).  For callers that report
+ * per-kernel figures and must name the kernel that ran.  No counterpart in the reference. */
+int l8_gemm_pick(int64_t M, int64_t N, int64_t K);
 
 #ifdef __cplusplus
 }

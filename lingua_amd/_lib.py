@@ -44,6 +44,7 @@ SIGNATURES = {
     "l8_rmsnorm_bwd_workspace": [_i64, _i64],
     "l8_gemm_algo_count": [],
     "l8_gemm_algo_name": [_int],
+    "l8_gemm_pick": [_i64, _i64, _i64],
 }
 _RETURNS_STR = {"l8_last_error", "l8_gemm_algo_name"}
 _RETURNS_I64 = {"l8_cast_rowwise_workspace", "l8_gemm_workspace", "l8_gemm_workspace_gave_up_offset", "l8_swiglu_workspace", "l8_rmsnorm_workspace", "l8_rmsnorm_bwd_workspace"}

@@ -222,30 +222,49 @@ __global__ __launch_bounds__(kRowBlock, (NCHW <= 4 ? 4 : (NCHW <= 8 ? 2 : 1))) v
 }
 
 // Folds the partial column maxima [n_slots, C] (bf16, one row per workgroup of a row-wise kernel) into
-// col_amax[C] (fp32 bit patterns), which is overwritten.  A workgroup owns kFoldPairs column pairs; its
-// kFoldGroups thread groups walk interleaved slots and meet in LDS: one launch, no atomics, nothing to
-// zero beforehand.
-constexpr int kFoldPairs = 64, kFoldGroups = 16;
-__global__ __launch_bounds__(kFoldPairs *kFoldGroups) void colmax_fold_kernel(const uint16_t *__restrict__ partials,
-                                                                               int n_slots, int C,
-                                                                               uint32_t *__restrict__ col_amax) {
-  __shared__ uint32_t red[kFoldGroups][kFoldPairs];
-  const int px = threadIdx.x % kFoldPairs, sy = threadIdx.x / kFoldPairs;
-  const int pair = blockIdx.x * kFoldPairs + px;
-  const bool live = pair * 2 < C;
-  uint32_t m = 0;
-  if (live) {
+// col_amax[C] (fp32 bit patterns), which is overwritten.  A workgroup owns 64 columns -- one 128-byte line of
+// every partial row -- and its 1024 threads read 16 bytes each from 128 rows at a time, so that a fold of a few
+// hundred rows is two to four loads per thread, all in flight at once (the kernel is pure latency: a few MB
+// read by a launch that lasts microseconds); the 128 row groups then meet in LDS.  One launch, no atomics,
+// nothing to zero beforehand.
+constexpr int kFoldCols = 64, kFoldThreads = 1024, kFoldRowGroups = kFoldThreads / 8;
+__global__ __launch_bounds__(kFoldThreads) void colmax_fold_kernel(const uint16_t *__restrict__ partials,
+                                                                   int n_slots, int C,
+                                                                   uint32_t *__restrict__ col_amax) {
+  __shared__ v4i red[kFoldRowGroups][8];
+  __shared__ uint32_t red2[8][32];
+  const int cc = threadIdx.x & 7;   // which 8 columns (16 bytes) of the 64
+  const int sg = threadIdx.x >> 3;  // row group
+  const int col = blockIdx.x * kFoldCols + cc * 8;
+  v4i m = {0, 0, 0, 0};
+  if (col < C) {
 #pragma unroll 4
-    for (int sl = sy; sl < n_slots; sl += kFoldGroups)
-      m = pk_absmax_u16(m, __builtin_nontemporal_load((const uint32_t *)(partials + (int64_t)sl * C) + pair));
-  }
-  red[sy][px] = m;
-  __syncthreads();
-  if (sy == 0 && live) {
+    for (int sl = sg; sl < n_slots; sl += kFoldRowGroups) {
+      const v4i v = __builtin_nontemporal_load((const v4i *)(partials + (int64_t)sl * C + col));
 #pragma unroll
-    for (int g = 1; g < kFoldGroups; ++g) m = pk_absmax_u16(m, red[g][px]);
-    col_amax[2 * pair] = (m & 0xffffu) << 16;  // bf16 -> fp32 bit patterns
-    col_amax[2 * pair + 1] = m & 0xffff0000u;
+      for (int k = 0; k < 4; ++k) m[k] = (int)pk_absmax_u16((uint32_t)m[k], (uint32_t)v[k]);
+    }
+  }
+  red[sg][cc] = m;
+  __syncthreads();
+  if (threadIdx.x < 256) {
+    const int pair = threadIdx.x & 31, part = threadIdx.x >> 5;  // 32 column pairs x 8 parts of 16 row groups
+    uint32_t mm = 0;
+#pragma unroll
+    for (int g = 0; g < kFoldRowGroups / 8; ++g)
+      mm = pk_absmax_u16(mm, reinterpret_cast<const uint32_t *>(&red[part * (kFoldRowGroups / 8) + g][0])[pair]);
+    red2[part][pair] = mm;
+  }
+  __syncthreads();
+  if (threadIdx.x < 32) {
+    uint32_t mm = 0;
+#pragma unroll
+    for (int part = 0; part < 8; ++part) mm = pk_absmax_u16(mm, red2[part][threadIdx.x]);
+    const int c = blockIdx.x * kFoldCols + threadIdx.x * 2;
+    if (c < C) {
+      col_amax[c] = (mm & 0xffffu) << 16;  // bf16 -> fp32 bit patterns
+      col_amax[c + 1] = mm & 0xffff0000u;
+    }
   }
 }
 
@@ -580,9 +599,8 @@ static int64_t rowwise_blocks(int64_t R, int64_t C, bool colmax) {
 }
 
 int fold_colmax(const void *partials, int64_t slots, int64_t C, float *col_amax, hipStream_t st) {
-  hipLaunchKernelGGL(colmax_fold_kernel, dim3((unsigned)((C / 2 + kFoldPairs - 1) / kFoldPairs)),
-                     dim3(kFoldPairs * kFoldGroups), 0, st, (const uint16_t *)partials, (int)slots, (int)C,
-                     (uint32_t *)col_amax);
+  hipLaunchKernelGGL(colmax_fold_kernel, dim3((unsigned)((C + kFoldCols - 1) / kFoldCols)), dim3(kFoldThreads), 0, st,
+                     (const uint16_t *)partials, (int)slots, (int)C, (uint32_t *)col_amax);
   L8_HIP(hipGetLastError());
   return L8_OK;
 }

@@ -512,12 +512,16 @@ __global__ __launch_bounds__(WM *WN * 64) void gemm_nt_kernel(const GemmArgs p) 
 // (the ring stays in use by the panel stream) and no barrier:
 //   * the matrix cores compute D[i = m][j = n'] (A rows on the first port);
 //   * LDS row tn*32 + j of a wave's 128-row span of the B panel holds the
-//     global B row 4*j + tn of that span (the permutation is applied on the
-//     global-address side of the direct-to-LDS loads, which is free), so that
-//     lane j owns, at the same accumulator index of its four tn tiles, the
-//     four CONSECUTIVE output columns 4*j .. 4*j+3;
-//   * one 8-byte store per lane then covers 256 contiguous bytes of a C row
-//     per half-wave (two rows per wave instruction, whole 128-byte lines).
+//     global B row 4*g(j) + tn of that span, g(j) = 2*(j & 15) + (j >> 4) (the
+//     permutation is applied on the global-address side of the direct-to-LDS
+//     loads, which is free), so that lane j owns, at the same accumulator
+//     index of its four tn tiles, the four CONSECUTIVE output columns
+//     4*g(j) .. 4*g(j)+3, and lanes j / j+16 own neighbouring groups;
+//   * two v_permlane16_swap per pair of rows hand the lanes 0..15 of every 32
+//     the first row (their own four columns and their partners' four) and the
+//     lanes 16..31 the second: one 16-byte store per lane then covers 256
+//     contiguous bytes of a C row per 16 lanes (four rows per wave instruction,
+//     whole 128-byte lines).
 // Work split: the tiles are dealt to the 8 XCDs in contiguous ranges of the
 // grouped order (as in the kernel above); inside an XCD, workgroup `loc`
 // takes tiles loc, loc + W, loc + 2W, ... of the range (W workgroups per XCD),
@@ -597,8 +601,8 @@ __global__ __launch_bounds__(256) void gemm_nt_stream_kernel(const GemmArgs p) {
   // lane l of a wave load fills LDS row l/8, position l%8 of an 8-row group; position p of LDS row r holds
   // chunk p ^ f(r), f(r) = (r & 7) ^ ((r >> 3) & 1).  Wave load i of a panel fills the LDS rows of group
   // g = wave * NL + i.  For the A panel LDS row = tile row.  For the B panel LDS row r = span*128 + tn*32 + j
-  // holds tile row span*128 + 4*j + tn: within a group (8 consecutive j) the rows are 4 apart, and the
-  // group's first row is span*128 + 4*(8*(g%4)) + (g%16)/4.
+  // holds tile row span*128 + 4*cg(j) + tn with cg(j) = 2*(j & 15) + (j >> 4): within a group (8 consecutive j)
+  // the rows are 8 apart, and the group's first row is span*128 + 64*(g & 1) + 4*((g >> 1) & 1) + (g%16)/4.
   // The per-lane constants of the K loop are formed afresh, from an opaque copy of the lane number, in front of
   // every tile's K loop: values that lived across the conversion of the C tile (the point of highest register
   // pressure) were the ones the allocator chose to spill, and it reloaded them inside the K loop.
@@ -612,8 +616,8 @@ __global__ __launch_bounds__(256) void gemm_nt_stream_kernel(const GemmArgs p) {
     chunk_odd = (lpos ^ lrow ^ 1) * 16;
     a_voff[0] = (uint32_t)(lrow * (int)p.lda + chunk_even);
     a_voff[1] = (uint32_t)(lrow * (int)p.lda + chunk_odd);
-    b_voff[0] = (uint32_t)(lrow * 4 * (int)p.ldb + chunk_even);
-    b_voff[1] = (uint32_t)(lrow * 4 * (int)p.ldb + chunk_odd);
+    b_voff[0] = (uint32_t)(lrow * 8 * (int)p.ldb + chunk_even);
+    b_voff[1] = (uint32_t)(lrow * 8 * (int)p.ldb + chunk_odd);
     const int l31 = l & 31, h = l >> 5;
     const int fr = (l31 & 7) ^ ((l31 >> 3) & 1);
 #pragma unroll
@@ -665,7 +669,7 @@ __global__ __launch_bounds__(256) void gemm_nt_stream_kernel(const GemmArgs p) {
       __builtin_amdgcn_raw_ptr_buffer_load_lds(ld_rsA, reinterpret_cast<lds_ptr_t>(dst), 16, a_voff[i & 1] | ((i & 1) ? m_odd : m_even),
                                                k0 + (wave * NL + i) * 8 * (int)p.lda, 0, 0);
     } else {
-      const int row = (wave >> 1) * 128 + 32 * (i & 3) + (wave & 1) * 2 + (i >> 2);
+      const int row = (wave >> 1) * 128 + 64 * (i & 1) + 4 * ((i >> 1) & 1) + (wave & 1) * 2 + (i >> 2);
       __builtin_amdgcn_raw_ptr_buffer_load_lds(ld_rsB, reinterpret_cast<lds_ptr_t>(dst), 16, b_voff[i & 1] | ((i & 1) ? m_odd : m_even),
                                                k0 + row * (int)p.ldb, 0, 0);
     }
@@ -673,6 +677,7 @@ __global__ __launch_bounds__(256) void gemm_nt_stream_kernel(const GemmArgs p) {
 
   // ---- LDS -> register fragment plan (as in the kernel above) ----
   const int l31 = lane & 31, h = lane >> 5;
+  const int cg = 2 * (l31 & 15) + (l31 >> 4);  // this lane's group of four output columns (of its wave's 32)
   const int a_base = wm * (TM * 32 * BK);
   const int b_base = wn * (TN * 32 * BK);
   typedef const __attribute__((address_space(3))) v4i *lds_v4i_ptr;
@@ -717,7 +722,7 @@ __global__ __launch_bounds__(256) void gemm_nt_stream_kernel(const GemmArgs p) {
   };
   // ---- C tile straight from the accumulators ----
   // acc[tm][tn][4*qd + e] of lane (l31, h) is C[m][n] with m = wm*128 + tm*32 + 8*qd + 4*h + e and
-  // n = wn*128 + 4*l31 + tn (tile coordinates).  The host launches this kernel only when every lane pair's
+  // n = wn*128 + 4*cg(l31) + tn (tile coordinates).  The host launches this kernel only when every lane pair's
   // eight columns are in or out as a whole and its 16-byte store is aligned: N % 8 == 0, ldc % 8 == 0, C
   // 16-byte aligned, row scales 16-byte and bias 8-byte aligned.
   // The scales (and the bias) of a tile are requested before its K loop, a handful of registers per lane: lane l
@@ -738,14 +743,14 @@ __global__ __launch_bounds__(256) void gemm_nt_stream_kernel(const GemmArgs p) {
     }
     if (p.sb_row) {
       const __amdgpu_buffer_rsrc_t rsSb = make_rsrc(p.sb + n0, sb_left < 0x7fffffff ? (uint32_t)sb_left : 0x7fffffffu);
-      seg_sb = __builtin_amdgcn_raw_buffer_load_b128(rsSb, (wn * 128 + 4 * l31) * 4, 0, 0);
+      seg_sb = __builtin_amdgcn_raw_buffer_load_b128(rsSb, (wn * 128 + 4 * cg) * 4, 0, 0);
     } else {
       const int bits = __float_as_int(p.sb[0]);
       seg_sb = v4i{bits, bits, bits, bits};
     }
     if constexpr (HAS_BIAS) {
       const __amdgpu_buffer_rsrc_t rsBias = make_rsrc(p.bias + n0, (uint32_t)((p.N - n0) * 2));
-      seg_bias = __builtin_amdgcn_raw_buffer_load_b64(rsBias, (wn * 128 + 4 * l31) * 2, 0, 0);
+      seg_bias = __builtin_amdgcn_raw_buffer_load_b64(rsBias, (wn * 128 + 4 * cg) * 2, 0, 0);
     }
   };
   // (A compute unit drains its stores at about 16 bytes per clock: the 128 KiB of a C tile keep it busy for some
@@ -759,13 +764,16 @@ __global__ __launch_bounds__(256) void gemm_nt_stream_kernel(const GemmArgs p) {
   [[maybe_unused]] __amdgpu_buffer_rsrc_t rs_p;
   [[maybe_unused]] int p_slot = 0;
   constexpr int P_AHEAD = 3;  // groups / pieces of the partial sum requested ahead of their use (their latency is long)
-  auto store_tile = [&](int m0, int n0, auto parts_tag) {
+  auto store_tile_as = [&](int m0, int n0, auto parts_tag, auto sbrow_tag) {
     constexpr bool PARTS = decltype(parts_tag)::value;
+    // SB_ROW false: one scale for all columns; it is folded into the row scales (two multiplications per lane and
+    // tile instead of one per element)
+    constexpr bool SB_ROW = decltype(sbrow_tag)::value;
     // Opaque copies: everything below would otherwise be hoisted out of the K loop as loop-invariant (row
     // offsets in scalar registers, per-lane addresses in vector registers) and held across it.
     int ldc2 = (int)p.ldc * 2;
     asm volatile("" : "+s"(ldc2));
-    int lane_col = wn * 128 + 4 * l31;
+    int lane_col = wn * 128 + 8 * (l31 & 15);  // first of the eight columns this lane stores
     asm volatile("" : "+v"(lane_col));
     const int64_t c_left = ((int64_t)(p.M - m0 - 1) * p.ldc + (p.N - n0)) * 2;
     const __amdgpu_buffer_rsrc_t rsC = make_rsrc(p.C + (int64_t)m0 * p.ldc + n0, c_left < 0x7fffffff ? (uint32_t)c_left : 0x7fffffffu);
@@ -785,7 +793,8 @@ __global__ __launch_bounds__(256) void gemm_nt_stream_kernel(const GemmArgs p) {
     // precomputed into 64 registers and spilled) and are waited for by hand: LDS operations return in order, so
     // "at most 4 outstanding" means that everything but the group requested last has arrived.
     const int sa_addr = 16 * h;  // byte address of lane 4*h
-    const int sa_regs[2] = {seg_sa[0], seg_sa[1]};
+    const int sa_regs[2] = {SB_ROW ? seg_sa[0] : __float_as_int(__int_as_float(seg_sa[0]) * sbv[0]),
+                            SB_ROW ? seg_sa[1] : __float_as_int(__int_as_float(seg_sa[1]) * sbv[0])};
     float sa_grp[2][4];
     auto request_row_scales = [&](int g, float (&dst)[4]) {  // g = tm * 4 + qd
       const int tm = g >> 2, qd = g & 3;
@@ -818,13 +827,12 @@ __global__ __launch_bounds__(256) void gemm_nt_stream_kernel(const GemmArgs p) {
       tq1 = __builtin_readcyclecounter();
       prof[8] += tq1 - tq0;
     }
-    // A store instruction costs the same whatever it carries, so neighbouring lanes pair up: of two consecutive
-    // rows, the even lane takes the first (its own four columns and the odd lane's four, 16 contiguous bytes)
-    // and the odd lane the second.  One instruction then writes four rows x 256 bytes.  Lanes whose columns lie
-    // beyond N store nothing (N % 8 == 0 here: a lane pair is in or out as a whole).
-    const int par = l31 & 1;
-    const uint32_t c_voff = (n0 + wn * 128 + 4 * (l31 & ~1) < p.N)
-                                ? (uint32_t)((4 * h + par) * ldc2 + (lane_col - 4 * par) * 2) : kOOB;
+    // A store instruction costs the same whatever it carries, so lanes j and j+16 pair up: of two consecutive
+    // rows, lane j takes the first (its own four columns and its partner's four, 16 contiguous bytes) and lane
+    // j+16 the second.  One instruction then writes four rows x 256 bytes.  Lanes whose columns lie beyond N
+    // store nothing (N % 8 == 0 here: a lane pair is in or out as a whole).
+    const int par = l31 >> 4;
+    const uint32_t c_voff = (n0 + lane_col < p.N) ? (uint32_t)((4 * h + par) * ldc2 + lane_col * 2) : kOOB;
     if (L8_GEMM_PROF) {
       __builtin_amdgcn_s_waitcnt(0x0070);  // the scales
       tq2 = __builtin_readcyclecounter();
@@ -857,7 +865,7 @@ __global__ __launch_bounds__(256) void gemm_nt_stream_kernel(const GemmArgs p) {
             for (int tn = 0; tn < TN; ++tn) {
               float a = acc_read(tm, tn, 4 * qd + e2 + r);
               if constexpr (PARTS) a = a + pbuf[g % (P_AHEAD + 1)][tn][e2 + r];  // ascending K
-              v[tn] = a * sa * sbv[tn];
+              v[tn] = SB_ROW ? a * sa * sbv[tn] : a * sa;
               if constexpr (HAS_BIAS) v[tn] += bv[tn];
             }
             typedef __bf16 bf2 __attribute__((ext_vector_type(2)));
@@ -865,11 +873,12 @@ __global__ __launch_bounds__(256) void gemm_nt_stream_kernel(const GemmArgs p) {
             o[r][0] = __builtin_bit_cast(int, lo);
             o[r][1] = __builtin_bit_cast(int, hi);
           }
-          // even lanes hand over their second row, odd lanes their first; quad_perm [1,0,3,2] swaps neighbours
-          const int give0 = par ? o[0][0] : o[1][0], give1 = par ? o[0][1] : o[1][1];
-          const int got0 = __builtin_amdgcn_update_dpp(0, give0, 0xB1, 0xF, 0xF, true);
-          const int got1 = __builtin_amdgcn_update_dpp(0, give1, 0xB1, 0xF, 0xF, true);
-          const v4i out = par ? v4i{got0, got1, o[1][0], o[1][1]} : v4i{o[0][0], o[0][1], got0, got1};
+          // lanes 0..15 of every 32 hand over their second row and get their partners' first, lanes 16..31 the
+          // other way round: v_permlane16_swap exchanges the odd rows of 16 lanes of its first operand with the
+          // even rows of its second
+          const auto s0 = __builtin_amdgcn_permlane16_swap((unsigned)o[0][0], (unsigned)o[1][0], false, false);
+          const auto s1 = __builtin_amdgcn_permlane16_swap((unsigned)o[0][1], (unsigned)o[1][1], false, false);
+          const v4i out = {(int)s0[0], (int)s1[0], (int)s0[1], (int)s1[1]};
           if (L8_GEMM_DIAG != 3 && !(L8_GEMM_DIAG == 8 && (qd & 1)))  // experiments: no stores (3), half of them (8)
             __builtin_amdgcn_raw_buffer_store_b128(out, rsC, c_voff, (row + e2) * ldc2, 2 /* streaming */);
           // one row pair at a time: left free, the scheduler reads a hundred accumulator registers ahead and the
@@ -888,6 +897,11 @@ __global__ __launch_bounds__(256) void gemm_nt_stream_kernel(const GemmArgs p) {
       for (int tn = 0; tn < TN; ++tn)
 #pragma unroll
         for (int v = 0; v < 16; ++v) acc[tm][tn][v] = 0.0f;
+  };
+
+  auto store_tile = [&](int m0, int n0, auto parts_tag) {
+    if (p.sb_row) store_tile_as(m0, n0, parts_tag, std::true_type{});
+    else store_tile_as(m0, n0, parts_tag, std::false_type{});
   };
 
   // ---- SK: exchange of partial sums for tiles whose K range is shared out ----
@@ -1193,6 +1207,13 @@ static int pick_algo(int64_t M, int64_t N, int64_t K) {
   const int64_t big_tiles = ((M + 255) / 256) * ((N + 255) / 256);
   if (big_tiles >= num_cus()) return 12;
   return 2;
+}
+
+// Host arithmetic only: the tile configuration `algo = 0` resolves to for this problem on the current device when
+// the operands allow every kernel (aligned, N % 8 == 0): what a caller that reports per-kernel figures names.
+extern "C" int l8_gemm_pick(int64_t M, int64_t N, int64_t K) {
+  L8_REQUIRE(M > 0 && N > 0 && K > 0, "l8_gemm_pick: empty problem");
+  return pick_algo(M, N, K);
 }
 
 // flags (one 4-byte word per workgroup, first 4 KiB) + one fp32 256x256 tile per workgroup of a persistent launch

@@ -293,6 +293,16 @@ def gemm_nt(qa: torch.Tensor, qb: torch.Tensor, sa: torch.Tensor, sb: torch.Tens
     return out
 
 
+def gemm_pick(M: int, N: int, K: int) -> Tuple[int, str]:
+    """(number, name) of the tile configuration that ``algo=0`` resolves to for an M x N x K problem on the current
+    device (aligned operands assumed)."""
+    lib = _lib.load()
+    algo = lib.l8_gemm_pick(M, N, K)
+    if algo <= 0:
+        _lib.check(algo, "l8_gemm_pick")
+    return algo, lib.l8_gemm_algo_name(algo).decode()
+
+
 def gemm_algos() -> Tuple[str, ...]:
     lib = _lib.load()
     return tuple(lib.l8_gemm_algo_name(i + 1).decode() for i in range(lib.l8_gemm_algo_count()))

@@ -24,4 +24,4 @@ def pytest_collection_modifyitems(config, items):
             item.add_marker(skip)
 
 
-from workloads import rel_l2, seeded_bf16  # noqa: E402,F401  (tests import them from here)
+from bench_workloads import rel_l2, seeded_bf16  # noqa: E402,F401  (tests import them from here)

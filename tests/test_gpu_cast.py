@@ -175,7 +175,7 @@ def test_colwise_nonfinite_columns():
     assert bits_equal(s[fin], so[fin])
 
 
-from workloads import outlier_stress_input  # noqa: E402
+from bench_workloads import outlier_stress_input  # noqa: E402
 
 
 def test_outlier_stress_full_size_rowwise_tensorwise_colwise():

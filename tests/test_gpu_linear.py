@@ -199,7 +199,7 @@ def test_config3_7b_mlp_forward_backward():
 def test_outlier_stress_rowwise_beats_tensorwise_on_the_linear():
     # config 4 at its full 16384 tokens: both recipes against the oracle's product of the very same bytes and scales
     # on a row sample, then the two recipes against each other
-    from workloads import outlier_stress_figures
+    from bench_workloads import outlier_stress_figures
     fig, t = outlier_stress_figures(16384)
     rows = torch.arange(0, 16384, 512).cuda()
     want_row = oracle.gemm_nt(t["qx"][rows].cpu().view(torch.uint8), t["qw"].cpu().view(torch.uint8), t["sx"][rows].cpu(), t["sw"].cpu())
@@ -218,7 +218,7 @@ def test_config5_llama_1b_training_step():
     # full Llama-1B-shaped step (25 layers, dim 2048, 16 heads, ffn 8192, vocab 128256, 4 x 4096 tokens), all block
     # linears fp8 row-wise, output head bf16; three linears are checked against the oracle through hooks
     from lingua_amd import convert_linears_to_fp8, Fp8Linear
-    from workloads import Llama, LLAMA_1B
+    from bench_workloads import Llama, LLAMA_1B
     torch.manual_seed(0)
     with torch.device("cuda"):
         model = Llama(**LLAMA_1B).to(torch.bfloat16)
@@ -317,7 +317,7 @@ def test_custom_ops_route_equals_the_autograd_function_and_compiles():
     (aot_eager: fake tensors + functionalisation + the registered autograd formula, no code generation)."""
     from lingua_amd import convert_linears_to_fp8, float8
     from lingua_amd import custom_ops
-    from workloads import FeedForward
+    from bench_workloads import FeedForward
     torch.manual_seed(6)
     holder = nn.ModuleDict({"feed_forward": FeedForward(256, 512).to(device="cuda", dtype=torch.bfloat16)})
     model = convert_linears_to_fp8(holder, "rowwise", r"feed_forward\.")["feed_forward"]
@@ -379,7 +379,7 @@ def test_mlp_step_is_bitwise_reproducible():
     """No result of the path depends on scheduling: the column amaxes are max-merged (order-free), every sum runs
     in a fixed order.  Two runs of the same MLP step give identical bits, drop-in and fused."""
     from lingua_amd import convert_linears_to_fp8
-    from workloads import FeedForward
+    from bench_workloads import FeedForward
     from lingua_amd.swiglu import Fp8FeedForward
     torch.manual_seed(12)
     holder = nn.ModuleDict({"feed_forward": FeedForward(512, 1536).to(device="cuda", dtype=torch.bfloat16)})
@@ -455,7 +455,7 @@ def test_inference_mode_matches_no_grad():
     reference generates that way): the shared-cast memo must step aside, results equal the no_grad ones."""
     from lingua_amd import convert_linears_to_fp8
     from lingua_amd.norm import fuse_rmsnorm
-    from workloads import TransformerBlock, rope_tables
+    from bench_workloads import TransformerBlock, rope_tables
     torch.manual_seed(3)
     holder = nn.ModuleDict({"layers": nn.ModuleList([TransformerBlock(256, 4, 64, 512).to(device="cuda", dtype=torch.bfloat16)])})
     x = seeded_bf16((2, 48, 256), seed=61).cuda()
@@ -512,7 +512,7 @@ def test_selective_checkpointing_saves_the_fp8_product():
     from functools import partial
     from torch.utils.checkpoint import CheckpointPolicy, checkpoint, create_selective_checkpoint_contexts
     from lingua_amd import convert_linears_to_fp8, float8, ops
-    from workloads import FeedForward
+    from bench_workloads import FeedForward
     torch.manual_seed(14)
     holder = nn.ModuleDict({"feed_forward": FeedForward(256, 512).to(device="cuda", dtype=torch.bfloat16)})
     mlp = convert_linears_to_fp8(holder, "rowwise", r"feed_forward\.")["feed_forward"]

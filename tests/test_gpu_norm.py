@@ -100,7 +100,7 @@ class _Block(torch.nn.Module):
 
     def __init__(self, dim):
         super().__init__()
-        from workloads import RMSNorm
+        from bench_workloads import RMSNorm
         self.attention_norm = RMSNorm(dim, EPS)
         self.wq = torch.nn.Linear(dim, dim, bias=False)
         self.wk = torch.nn.Linear(dim, dim // 2, bias=False)
@@ -163,7 +163,7 @@ def test_small_llama_with_fused_gate_and_norms_matches_the_drop_in_model():
     models are not compared with each other directly: each gradient of the fused model must be as close to the
     bf16 model's as the drop-in model's is (within a quarter more), and the losses must agree."""
     from lingua_amd import convert_linears_to_fp8
-    from workloads import Llama
+    from bench_workloads import Llama
     from lingua_amd.norm import Fp8RMSNorm, fuse_rmsnorm
     from lingua_amd.swiglu import Fp8FeedForward, fuse_feed_forward
     cfg = dict(n_layers=3, dim=512, n_heads=4, ffn_dim=1536, vocab=1000)
@@ -209,7 +209,7 @@ def test_fused_feed_forward_takes_the_norm_output_already_quantised():
     from lingua_amd import float8, ops
     from lingua_amd.norm import Fp8RMSNorm
     from lingua_amd.swiglu import Fp8FeedForward
-    from workloads import FeedForward
+    from bench_workloads import FeedForward
     torch.manual_seed(4)
     ff = FeedForward(512, 1024).to(device="cuda", dtype=torch.bfloat16)
     norm = Fp8RMSNorm(512, 1e-5).to(device="cuda", dtype=torch.bfloat16)

@@ -7,7 +7,7 @@ import pytest
 import torch
 
 from conftest import rel_l2, seeded_bf16
-import workloads
+import bench_workloads as workloads
 
 pytestmark = pytest.mark.gpu
 

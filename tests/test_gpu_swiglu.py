@@ -145,7 +145,7 @@ def test_argument_errors():
 
 
 def _mlps(dim, ffn, seed):
-    import workloads as callers
+    import bench_workloads as callers
     from lingua_amd import convert_linears_to_fp8
     from lingua_amd.swiglu import Fp8FeedForward, fuse_feed_forward
     torch.manual_seed(seed)

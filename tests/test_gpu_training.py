@@ -13,7 +13,7 @@ STEPS = 40
 
 def _train(kind):
     from lingua_amd import convert_linears_to_fp8, float8
-    from workloads import Llama
+    from bench_workloads import Llama
     from lingua_amd.norm import fuse_rmsnorm
     from lingua_amd.swiglu import fuse_feed_forward
     with torch.device("cuda"):
@@ -69,7 +69,7 @@ def test_activation_checkpointing_reproduces_the_plain_backward(fused):
     The kernels are deterministic, so loss and every gradient are bit-identical to the run without it."""
     from torch.utils.checkpoint import checkpoint
     from lingua_amd import convert_linears_to_fp8
-    from workloads import Llama, rope_tables
+    from bench_workloads import Llama, rope_tables
     from lingua_amd.norm import fuse_rmsnorm
     from lingua_amd.swiglu import fuse_feed_forward
     with torch.device("cuda"):
