@@ -69,7 +69,7 @@ def _check_usage(usage) -> None:
     unread = [name for name, u in stream.items() if "ScratchSize" not in u or "VGPRs Spill" not in u]
     if unread:
         raise RuntimeError("resource remarks without scratch / spill figures for:\n  " + "\n  ".join(unread))
-    bad = [f"{name}: {u}" for name, u in stream.items() if u["ScratchSize"] or u["VGPRs Spill"]]
+    bad = [f"{name}: {u}" for name, u in stream.items() if (u["ScratchSize"] or u["VGPRs Spill"])]
     if bad:
         raise RuntimeError("the persistent GEMM kernel must not use scratch memory:\n  " + "\n  ".join(bad))
 

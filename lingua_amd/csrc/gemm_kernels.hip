@@ -82,6 +82,21 @@ L8_DEV __amdgpu_buffer_rsrc_t make_rsrc(const void *p, uint32_t bytes) {
 }
 #endif
 
+// 16-byte-per-lane buffer store with a scalar-register offset, followed by two wait states.  A vector-ALU write to
+// one of the store's data registers right behind it can reach the register before the store has read it: with two
+// waves per SIMD the eight-wave kernel stored, now and then, the next row pair's values in 4 of 64 lanes (found by
+// the exact-integer tests; two wait states cure it, which is what the compiler's hazard recognizer inserts behind
+// stores of more than 8 bytes -- except behind buffer stores whose soffset is a register, like these, which an old
+// rule exempts).  Every such store in this file goes through here.
+#if defined(__HIP_DEVICE_COMPILE__)
+template <int AUX>
+L8_DEV void store16_aux(v4i data, __amdgpu_buffer_rsrc_t rs, uint32_t voff, int soff) {
+  __builtin_amdgcn_raw_buffer_store_b128(data, rs, voff, soff, AUX);
+  asm volatile("s_nop 1");
+}
+#endif
+#define store16(data, rs, voff, soff, aux) store16_aux<aux>(data, rs, voff, soff)
+
 [[maybe_unused]] constexpr uint32_t kOOB = 0x80000000u;
 // cache policy of a buffer access that must be coherent over the whole device (sc0 | sc1)
 [[maybe_unused]] constexpr int kCoherent = 1 | 16;
@@ -528,10 +543,16 @@ __global__ __launch_bounds__(WM *WN * 64) void gemm_nt_kernel(const GemmArgs p) 
 // so the workgroups resident on an XCD always work on W consecutive tiles of
 // the grouped order and share their panels in that XCD's L2.
 // ---------------------------------------------------------------------------
-template <int GROUP_M, bool HAS_BIAS, bool SK = false>
-__global__ __launch_bounds__(256) void gemm_nt_stream_kernel(const GemmArgs p) {
+template <int GROUP_M, bool HAS_BIAS, bool SK = false, int NW = 4>
+__global__ __launch_bounds__(NW * 64) void gemm_nt_stream_kernel(const GemmArgs p) {
 #if defined(__HIP_DEVICE_COMPILE__)
-  constexpr int BM = 256, BN = 256, BK = 128, NW = 4, TM = 4, TN = 4, R = 5;
+  // NW = 4: one wave per SIMD, 128x128 per wave (the least LDS traffic per flop); NW = 8: two waves per SIMD,
+  // 64x128 per wave (while one of them waits -- for the port of the vector memory unit, for LDS, at the barrier --
+  // the other one's MFMAs keep the matrix core busy; half the stores per wave in the epilogue; 1.5 x the LDS reads)
+  static_assert(NW == 4 || NW == 8, "four or eight waves");
+  static_assert(!SK || NW == 4, "the shared-K exchange is written for four waves");
+  constexpr int BM = 256, BN = 256, BK = 128, TM = 16 / NW, TN = 4, R = 5;
+  constexpr int WROWS = TM * 32;  // rows of the tile per wave
   constexpr int UNIT = BM * BK;    // one ring slot: the A or the B panel of one K tile
   constexpr int NL = BM / 8 / NW;  // 1 KiB wave loads (8 rows x 128 B) per panel per wave
   constexpr int PEND = NL;         // in flight at the barrier of a trip: the unit requested in its first half
@@ -669,15 +690,14 @@ __global__ __launch_bounds__(256) void gemm_nt_stream_kernel(const GemmArgs p) {
       __builtin_amdgcn_raw_ptr_buffer_load_lds(ld_rsA, reinterpret_cast<lds_ptr_t>(dst), 16, a_voff[i & 1] | ((i & 1) ? m_odd : m_even),
                                                k0 + (wave * NL + i) * 8 * (int)p.lda, 0, 0);
     } else {
-      const int row = (wave >> 1) * 128 + 64 * (i & 1) + 4 * ((i >> 1) & 1) + (wave & 1) * 2 + (i >> 2);
+      const int g = wave * NL + i;  // 8-row group of the panel's LDS image
+      const int row = (g >> 4) * 128 + 64 * (g & 1) + 4 * ((g >> 1) & 1) + ((g & 15) >> 2);
       __builtin_amdgcn_raw_ptr_buffer_load_lds(ld_rsB, reinterpret_cast<lds_ptr_t>(dst), 16, b_voff[i & 1] | ((i & 1) ? m_odd : m_even),
                                                k0 + row * (int)p.ldb, 0, 0);
     }
   };
 
   // ---- LDS -> register fragment plan (as in the kernel above) ----
-  const int l31 = lane & 31, h = lane >> 5;
-  const int cg = 2 * (l31 & 15) + (l31 >> 4);  // this lane's group of four output columns (of its wave's 32)
   const int a_base = wm * (TM * 32 * BK);
   const int b_base = wn * (TN * 32 * BK);
   typedef const __attribute__((address_space(3))) v4i *lds_v4i_ptr;
@@ -716,28 +736,38 @@ __global__ __launch_bounds__(256) void gemm_nt_stream_kernel(const GemmArgs p) {
   // given plain reads, the register allocator moves the whole accumulator set into ordinary vector registers in
   // front of the conversion of the C tile and pays for it with spills inside the K loop.
   auto acc_read = [&](int tm, int tn, int i) -> float {
-    float x;
-    asm volatile("v_accvgpr_read_b32 %0, %1" : "=v"(x) : "a"(acc[tm][tn][i]));
-    return x;
+    if constexpr (NW == 8) {
+      return acc[tm][tn][i];  // 128 accumulators: the allocator may keep them in ordinary registers
+    } else {
+      float x;
+      asm volatile("v_accvgpr_read_b32 %0, %1" : "=v"(x) : "a"(acc[tm][tn][i]));
+      return x;
+    }
   };
   // ---- C tile straight from the accumulators ----
-  // acc[tm][tn][4*qd + e] of lane (l31, h) is C[m][n] with m = wm*128 + tm*32 + 8*qd + 4*h + e and
+  // acc[tm][tn][4*qd + e] of lane (l31, h) is C[m][n] with m = wm*WROWS + tm*32 + 8*qd + 4*h + e and
   // n = wn*128 + 4*cg(l31) + tn (tile coordinates).  The host launches this kernel only when every lane pair's
   // eight columns are in or out as a whole and its 16-byte store is aligned: N % 8 == 0, ldc % 8 == 0, C
   // 16-byte aligned, row scales 16-byte and bias 8-byte aligned.
   // The scales (and the bias) of a tile are requested before its K loop, a handful of registers per lane: lane l
-  // holds the A scales of tile rows wm*128 + l and + 64 + l (handed to the lanes that need them by lane
+  // holds the A scales of tile rows wm*WROWS + l and (four waves) + 64 + l (handed to the lanes that need them by lane
   // permutes at the end) and the B scales / bias of its own four columns.  Requested among the stores of the
   // tile they would make their consumer wait for every store ahead of them (the counter retires in order).
   int seg_sa[2] = {0, 0};
   v4i seg_sb = {0, 0, 0, 0};
   [[maybe_unused]] v2i seg_bias = {0, 0};
   auto load_scales = [&](int m0, int n0) {
+    // lane-derived values are formed afresh from an opaque copy of the lane number wherever a tile's prologue or
+    // epilogue needs them, so that none of them lives across a K loop
+    int l = lane;
+    asm volatile("" : "+v"(l));
+    const int l31 = l & 31;
+    const int cg = 2 * (l31 & 15) + (l31 >> 4);  // this lane's group of four output columns (of its wave's 32)
     const int64_t sa_left = (int64_t)(p.M - m0) * 4, sb_left = (int64_t)(p.N - n0) * 4;
     if (p.sa_row) {
       const __amdgpu_buffer_rsrc_t rsSa = make_rsrc(p.sa + m0, sa_left < 0x7fffffff ? (uint32_t)sa_left : 0x7fffffffu);
-      seg_sa[0] = __builtin_amdgcn_raw_buffer_load_b32(rsSa, (wm * 128 + lane) * 4, 0, 0);
-      seg_sa[1] = __builtin_amdgcn_raw_buffer_load_b32(rsSa, (wm * 128 + 64 + lane) * 4, 0, 0);
+      seg_sa[0] = __builtin_amdgcn_raw_buffer_load_b32(rsSa, (wm * WROWS + l) * 4, 0, 0);
+      if constexpr (TM == 4) seg_sa[1] = __builtin_amdgcn_raw_buffer_load_b32(rsSa, (wm * WROWS + 64 + l) * 4, 0, 0);
     } else {
       seg_sa[0] = seg_sa[1] = __float_as_int(p.sa[0]);
     }
@@ -773,6 +803,9 @@ __global__ __launch_bounds__(256) void gemm_nt_stream_kernel(const GemmArgs p) {
     // offsets in scalar registers, per-lane addresses in vector registers) and held across it.
     int ldc2 = (int)p.ldc * 2;
     asm volatile("" : "+s"(ldc2));
+    int l = lane;
+    asm volatile("" : "+v"(l));
+    const int l31 = l & 31, h = l >> 5;
     int lane_col = wn * 128 + 8 * (l31 & 15);  // first of the eight columns this lane stores
     asm volatile("" : "+v"(lane_col));
     const int64_t c_left = ((int64_t)(p.M - m0 - 1) * p.ldc + (p.N - n0)) * 2;
@@ -787,7 +820,7 @@ __global__ __launch_bounds__(256) void gemm_nt_stream_kernel(const GemmArgs p) {
       bv[2] = bf16_bits_to_f32((uint32_t)seg_bias[1] & 0xffffu);
       bv[3] = bf16_bits_to_f32((uint32_t)seg_bias[1] >> 16);
     }
-    // Row scale of tile row wm*128 + r: lane r % 64 of seg_sa[r / 64]; a lane needs r = tm*32 + 8*qd + 4*h + e.
+    // Row scale of tile row wm*WROWS + r: lane r % 64 of seg_sa[r / 64]; a lane needs r = tm*32 + 8*qd + 4*h + e.
     // The lane permutes of the next (tm, qd) group are in flight while the current group is converted.  They are
     // written as assembly for the immediate offset (as plain address arithmetic the 64 addresses were
     // precomputed into 64 registers and spilled) and are waited for by hand: LDS operations return in order, so
@@ -842,7 +875,7 @@ __global__ __launch_bounds__(256) void gemm_nt_stream_kernel(const GemmArgs p) {
     for (int tm = 0; tm < TM; ++tm) {
 #pragma unroll
       for (int qd = 0; qd < 4; ++qd) {
-        const int row = wm * 128 + tm * 32 + 8 * qd;  // + 4*h + e
+        const int row = wm * WROWS + tm * 32 + 8 * qd;  // + 4*h + e
         const int g = tm * 4 + qd;
         float(&sa_cur)[4] = sa_grp[g & 1];
         if constexpr (PARTS) {
@@ -880,7 +913,7 @@ __global__ __launch_bounds__(256) void gemm_nt_stream_kernel(const GemmArgs p) {
           const auto s1 = __builtin_amdgcn_permlane16_swap((unsigned)o[0][1], (unsigned)o[1][1], false, false);
           const v4i out = {(int)s0[0], (int)s1[0], (int)s0[1], (int)s1[1]};
           if (L8_GEMM_DIAG != 3 && !(L8_GEMM_DIAG == 8 && (qd & 1)))  // experiments: no stores (3), half of them (8)
-            __builtin_amdgcn_raw_buffer_store_b128(out, rsC, c_voff, (row + e2) * ldc2, 2 /* streaming */);
+            store16(out, rsC, c_voff, (row + e2) * ldc2, 2 /* streaming */);
           // one row pair at a time: left free, the scheduler reads a hundred accumulator registers ahead and the
           // register pressure of this conversion makes the allocator spill values the K loop uses in every trip
           __builtin_amdgcn_sched_barrier(0);
@@ -924,7 +957,7 @@ __global__ __launch_bounds__(256) void gemm_nt_stream_kernel(const GemmArgs p) {
 #pragma unroll
         for (int qd = 0; qd < 4; ++qd) {
           const v4f v = {acc_read(tm, tn, 4 * qd), acc_read(tm, tn, 4 * qd + 1), acc_read(tm, tn, 4 * qd + 2), acc_read(tm, tn, 4 * qd + 3)};
-          __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(v4i, v), rs, voff, piece_off(slot, (tm * TN + tn) * 4 + qd), kCoherent);
+          store16(__builtin_bit_cast(v4i, v), rs, voff, piece_off(slot, (tm * TN + tn) * 4 + qd), kCoherent);
         }
         __builtin_amdgcn_sched_barrier(0);
       }
@@ -989,7 +1022,7 @@ __global__ __launch_bounds__(256) void gemm_nt_stream_kernel(const GemmArgs p) {
   // group: the fragment addresses of a half are formed in the middle of the half before (ad_a for the first half,
   // ad_b for the second), and the LDS reads of a half are all issued in its first RD groups, so that the wait for
   // them at the end of the half (barrier, loop top) finds them landed.
-  constexpr int RD = L8_READ_GROUPS, G_ADDR = 8;
+  constexpr int RD = L8_READ_GROUPS < S1 ? L8_READ_GROUPS : S1, G_ADDR = N_MMA / 2;
   static_assert(RD >= NF / 2 && RD <= S1 && RD <= S2 - STRADDLE && G_ADDR < S1, "group layout");
   uint32_t ad_a[4], ad_b[4];
   frag_addrs(0, 1, 1, ad_a);
@@ -1166,6 +1199,7 @@ template __global__ void gemm_nt_stream_kernel<2, false>(const GemmArgs);
 template __global__ void gemm_nt_stream_kernel<2, true>(const GemmArgs);
 template __global__ void gemm_nt_stream_kernel<16, false>(const GemmArgs);
 template __global__ void gemm_nt_stream_kernel<16, true>(const GemmArgs);
+template __global__ void gemm_nt_stream_kernel<4, false, false, 8>(const GemmArgs);
 
 static const Algo kAlgos[] = {
     L8_ALGO_LIST(L8_ALGO_ROW)
@@ -1182,6 +1216,10 @@ static const Algo kAlgos[] = {
        clock higher, which recovers most of what the idle ones lose. */
     {"stream_mt2x2w_4x4t_r5_g4_sk", gemm_nt_stream_kernel<4, false>, 256, 256, 256, 5 * 256 * 128, true, gemm_nt_stream_kernel<4, true>,
      gemm_nt_stream_kernel<4, false, true>},
+    /* 16: algo 12 with eight waves (two per SIMD, 64x128 each), kept for the comparison: measured 1-2 % ahead of
+       algo 12 at K = 4096 and 2-4 % behind it at K >= 8192 (1.5 x the LDS reads); a product with a bias takes the
+       plain kernel (the bias instantiation would not fit the 256 registers of a wave without spills) */
+    {"stream_mt4x2w_2x4t_r5_g4", gemm_nt_stream_kernel<4, false, false, 8>, 256, 256, 512, 5 * 256 * 128, true, nullptr, nullptr},
 };
 constexpr int kNumAlgos = sizeof(kAlgos) / sizeof(kAlgos[0]);
 
@@ -1201,11 +1239,13 @@ static int pick_plain_big(int64_t K) { return K >= 4096 ? 5 : 3; }
 
 static int pick_algo(int64_t M, int64_t N, int64_t K) {
   // large problems: the persistent kernel (measured 2-11 % ahead of the plain ones on every shape with at
-  // least one 256x256 tile per compute unit; groups of 4 tile rows ahead of groups of 8 by 1-3 %); problems
-  // that would leave most of the chip idle with big tiles: 128x128 tiles
+  // least one 256x256 tile per compute unit; groups of 4 tile rows ahead of groups of 8 by 1-3 %), also when
+  // the big tiles leave up to 7/16 of the compute units idle (measured with K = 2048 .. 16384: 144 to 240
+  // tiles on 256 compute units run 10-25 % faster than with 128x128 tiles, 128 tiles and fewer 15-45 % slower);
+  // problems that would leave more of the chip idle with big tiles: 128x128 tiles
   (void)K;
   const int64_t big_tiles = ((M + 255) / 256) * ((N + 255) / 256);
-  if (big_tiles >= num_cus()) return 12;
+  if (big_tiles * 16 >= (int64_t)num_cus() * 9) return 12;
   return 2;
 }
 
@@ -1278,7 +1318,8 @@ static int gemm_nt_impl(const void *A, const void *B, int64_t M, int64_t N, int6
     // at a time; operands that do not allow that go to the plain kernel with the same tile shape
     const bool ok = N % 8 == 0 && ldc % 8 == 0 && ((uintptr_t)C % 16) == 0 && ldc < (1LL << 22) &&
                     (sa_mode != L8_SCALE_ROW || ((uintptr_t)sa % 16) == 0) &&
-                    (sb_mode != L8_SCALE_ROW || ((uintptr_t)sb % 16) == 0) && (bias == nullptr || ((uintptr_t)bias % 8) == 0);
+                    (sb_mode != L8_SCALE_ROW || ((uintptr_t)sb % 16) == 0) &&
+                    (bias == nullptr || (((uintptr_t)bias % 8) == 0 && kAlgos[algo - 1].fn_bias != nullptr));
     if (!ok) algo = pick_plain_big(K);
   }
   const Algo &al = kAlgos[algo - 1];

@@ -21,7 +21,7 @@ def fp8(t):
     return t.to(torch.float8_e4m3fn)
 
 
-ALGOS = list(range(0, 16))
+ALGOS = list(range(0, 17))
 SHAPES_EXACT = [(1, 1, 16), (32, 32, 64), (256, 256, 128), (256, 256, 256), (300, 200, 144), (257, 513, 272),
                 (64, 1000, 48), (1000, 24, 208), (512, 768, 240)]
 
