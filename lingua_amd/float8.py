@@ -153,17 +153,25 @@ def matmul(first, amax_first, second_t, amax_second_t, bias, use_fast_accum: boo
 
 
 class _LastCast:
-    """One-entry memo of the last activation quantised.  A lookup hits when it sees the same
-    memory (pointer, shape, strides, dtype, stream) at the same version counter AND comes from
-    a consumer (weight) that has not used the entry yet: the same weight asking again means a
-    new pass over the model, which quantises afresh.  The entry keeps the tensor alive, so its
-    address cannot be handed to another tensor while it is cached; the forward entry is dropped
-    by the first backward that runs and the backward entry by the next forward."""
+    """Memo of the last activation quantised, one entry per (device, stream): two models that step on two streams
+    (or two devices) do not evict each other.  A lookup hits when it sees the same memory (pointer, shape,
+    strides, dtype) at the same version counter AND comes from a consumer (weight) that has not used the entry
+    yet: the same weight asking again means a new pass over the model, which quantises afresh.  An entry keeps
+    its tensor alive, so the address cannot be handed to another tensor while it is cached; a stream's forward
+    entry is dropped by the first backward that runs on it and its backward entry by the next forward.  At most
+    ``MAX_SLOTS`` streams are remembered (the oldest entry goes first)."""
+
+    MAX_SLOTS = 16
 
     def __init__(self):
-        # one tuple (key, tensor kept alive, value, consumers), replaced as a whole: a reader on another
-        # thread (forward and autograd threads both come here) sees either the old entry or the new one
-        self.entry = None
+        # slot -> (key, tensor kept alive, value, consumers); tuples are replaced as a whole and dict updates are
+        # atomic under the interpreter lock: a reader on another thread (forward and autograd threads both come
+        # here) sees either the old entry or the new one
+        self.entries = {}
+
+    @staticmethod
+    def _slot(t):
+        return (t.device.index, torch.cuda.current_stream(t.device).cuda_stream)
 
     @staticmethod
     def _key(t):
@@ -171,21 +179,34 @@ class _LastCast:
                 torch.cuda.current_stream(t.device).cuda_stream)
 
     def get(self, t, user):
-        entry = self.entry
         # inference tensors have no version counter: nothing would show a write, so they are never shared
-        if entry is None or t.is_inference() or user in entry[3] or entry[0] != self._key(t):
+        if t.is_inference():
+            return None
+        entry = self.entries.get(self._slot(t))
+        if entry is None or user in entry[3] or entry[0] != self._key(t):
             return None
         entry[3].add(user)
         return entry[2]
 
     def put(self, t, value, user):
+        slot = self._slot(t)
         if t.is_inference():
-            self.entry = None
+            self.entries.pop(slot, None)
             return
-        self.entry = (self._key(t), t, value, {user})
+        self.entries.pop(slot, None)          # re-inserted below: the dict's order is the order of last use
+        while len(self.entries) >= self.MAX_SLOTS:
+            try:
+                self.entries.pop(next(iter(self.entries)), None)
+            except (StopIteration, RuntimeError):
+                break
+        self.entries[slot] = (self._key(t), t, value, {user})
 
-    def clear(self):
-        self.entry = None
+    def clear(self, like=None):
+        """Drops the entry of the device and current stream of ``like``, or every entry (``like=None``)."""
+        if like is None:
+            self.entries.clear()
+        elif like.is_cuda:
+            self.entries.pop(self._slot(like), None)
 
 
 _fwd_cast = _LastCast()   # a -> (qa, sa, a_col_amax | None)
@@ -276,7 +297,7 @@ def linear_forward(a, b_t, bias, need_wgrad_stats: bool, gemm_algo: int):
     if a.dtype != torch.bfloat16 or b_t.dtype != torch.bfloat16:
         raise RuntimeError(f"Fp8LinearFn: bf16 input and weight required, got {a.dtype} and {b_t.dtype}")
     # column amaxes of `a` fall out of the row-wise pass; wgrad wants them
-    _bwd_cast.clear()
+    _bwd_cast.clear(a)
     hit = _fwd_cast.get(a, b_t.data_ptr()) if config.share_input_casts else None
     if hit is not None and (hit[2] is not None or not need_wgrad_stats):
         qa, sa, a_col_amax = hit
@@ -312,8 +333,8 @@ def linear_backward(grad_out, a, b_t, amax_b_t, a_col_amax, need_a: bool, need_b
     if grad_out.dtype != torch.bfloat16:
         raise RuntimeError(f"Fp8LinearFn.backward: bf16 grad_out required, got {grad_out.dtype}")
     fp8_wgrad = fp8_wgrad and need_b
-    _fwd_cast.clear()
-    _fwd_tcast.clear()
+    _fwd_cast.clear(grad_out)
+    _fwd_tcast.clear(grad_out)
     if a is None and need_b and not (fp8_wgrad and a_tcast is not None):
         raise RuntimeError("Fp8LinearFn.backward: the bf16 input was not saved and no quantised copy stands in for it")
 

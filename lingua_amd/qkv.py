@@ -39,7 +39,7 @@ class Fp8QKVFn(torch.autograd.Function):
                 raise RuntimeError(f"Fp8QKVFn: bf16 input and weights required, got {t.dtype}")
         cfg = f8.config
         need_stats = cfg.fp8_wgrad and any(w.requires_grad for w in ws)
-        f8._bwd_cast.clear()
+        f8._bwd_cast.clear(x)
         hit = f8._fwd_cast.get(x, ("qkv", wq.data_ptr())) if cfg.share_input_casts else None
         if hit is not None and (hit[2] is not None or not need_stats):
             qx, sx, x_col = hit
