@@ -23,8 +23,6 @@ import time
 ROOT = os.path.dirname(os.path.abspath(__file__))
 if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
-if os.path.join(ROOT, "tests") not in sys.path:
-    sys.path.append(os.path.join(ROOT, "tests"))   # tests/workloads.py: the stand-in Llama and the seeded inputs
 
 DIM, FFN, TOKENS = 4096, 11008, 16384
 STEP_FLOP = 18 * TOKENS * DIM * FFN          # 9 GEMMs x 2*M*N*K
@@ -245,8 +243,25 @@ def config_figures(torch, dev, iters=20, warm=5):
         lin.weight.copy_(seeded_bf16((2048, 2048), 0.02, seed=1).to(dev))
         x1 = seeded_bf16((4096, 2048), 1.0, seed=0).to(dev)
         ms = clock(lambda: lin(x1))
-        res["config1_linear_forward"] = {"ms": round(ms, 4), "TFLOP/s": round(2 * 4096 * 2048 * 2048 / (ms * 1e-3) / 1e12, 1),
-                                         "what": "x [4096,2048] @ W [2048,2048]^T, both casts + GEMM per call"}
+        flop1 = 2 * 4096 * 2048 * 2048
+        res["config1_linear_forward"] = {"ms": round(ms, 4), "TFLOP/s": round(flop1 / (ms * 1e-3) / 1e12, 1),
+                                         "what": "x [4096,2048] @ W [2048,2048]^T, both casts + GEMM per call, eager: three "
+                                                 "launches of 5-20 us each, so the host's launch path is what is timed"}
+        # the same call replayed from a captured HIP graph: what the GPU needs for it
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            lin(x1)
+        torch.cuda.current_stream().wait_stream(side)
+        torch.cuda.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            y_graph = lin(x1)
+        ms = clock(graph.replay)
+        assert torch.equal(y_graph, lin(x1))
+        res["config1_linear_forward"]["graph_replay_ms"] = round(ms, 4)
+        res["config1_linear_forward"]["graph_replay_TFLOP/s"] = round(flop1 / (ms * 1e-3) / 1e12, 1)
+        del graph, y_graph
         mlp = make_mlp(torch, nn, 2048, 8192, dev)
         mlp = convert_linears_to_fp8(nn.ModuleDict({"layers": nn.ModuleList([mlp])}), "rowwise", r"layers\.[0-9]+\.")["layers"][0]
         x2 = seeded_bf16((32768, 2048), 1.0, seed=2).to(dev)
