@@ -947,7 +947,6 @@ __global__ __launch_bounds__(NW * 64) void gemm_nt_stream_kernel(const GemmArgs 
     return make_rsrc(p.sk_partials + (int64_t)slot * (BM * BN), BM * BN * 4);
   };
   [[maybe_unused]] auto write_partial = [&](int slot) {
-    constexpr int N_PIECES = TM * TN * 4;
     const __amdgpu_buffer_rsrc_t rs = partial_rsrc(slot);
     const int voff = lane * 16;
 #pragma unroll
@@ -1013,7 +1012,7 @@ __global__ __launch_bounds__(NW * 64) void gemm_nt_stream_kernel(const GemmArgs 
   // MFMAs of step 1 + LDS reads of the next K tile's step 0 + requests for the matching B panel.
   constexpr int N_MMA = TM * TN, NF = TM + TN;
   constexpr int STRADDLE = L8_STRADDLE < N_MMA - 2 ? L8_STRADDLE : 0;
-  constexpr int S1 = N_MMA - STRADDLE, S2 = N_MMA + STRADDLE, SR = N_MMA - 2;
+  constexpr int S1 = N_MMA - STRADDLE, S2 = N_MMA + STRADDLE;
   int s0 = 0;  // ring slot of the A panel of the K tile being multiplied
   // WAIT = the count of the wait in front of the barrier: everything older than the WAIT youngest requests must
   // have landed.
