@@ -144,6 +144,19 @@ def cpu_baseline(torch, sample_tokens):
     rt.matmul(x4, x4.abs().amax().reshape(1, 1), w4, w4.abs().amax().reshape(1, 1))
     c4 = time.perf_counter() - t0
     del x4, w4
+    # configs[4]: the seven fp8 linears of one Llama-1B block, forward + backward on the step's 16384 tokens, one repetition
+    # (the block's attention, norms and the head are not part of the path and are left out; a step has 25 such blocks)
+    t5 = 0.0
+    for n_out, n_in, count in ((2048, 2048, 4), (8192, 2048, 2), (2048, 8192, 1)):
+        a5 = torch.randn(TOKENS, n_in, generator=g).to(torch.bfloat16)
+        g5 = (torch.randn(TOKENS, n_out, generator=g) * 1e-2).to(torch.bfloat16)
+        w5 = (torch.randn(n_out, n_in, generator=g) * 0.02).to(torch.bfloat16)
+        t0 = time.perf_counter()
+        for _ in range(count):
+            rt.linear_fwd_bwd(a5, w5, g5)
+        t5 += time.perf_counter() - t0
+    del a5, g5, w5
+    flop5 = 6 * TOKENS * (4 * 2048 * 2048 + 3 * 2048 * 8192)
     return {
         "value": round(flop / dt / 1e12, 4),
         "unit": "TFLOP/s",
@@ -158,6 +171,11 @@ def cpu_baseline(torch, sample_tokens):
         "config4_outlier_stress_linear": {"value": round(2 * 2 * TOKENS * DIM * FFN / c4 / 1e12, 4), "unit": "TFLOP/s", "s": round(c4, 2),
                                           "sample": "4096 -> 11008 linear forward on the outlier-stress activations, row-wise + "
                                                     "tensor-wise, 16384 tokens, one repetition"},
+        "config5_llama1b_block_linears": {"value": round(flop5 / t5 / 1e12, 4), "unit": "TFLOP/s", "s": round(t5, 2),
+                                          "extrapolated_s_per_step": round(25 * t5, 1),
+                                          "sample": "the 7 fp8 linears of ONE Llama-1B block (wq, wk, wv, wo, w1, w3, w2), forward + "
+                                                    "backward, 16384 tokens, one repetition; extrapolated_s_per_step = 25 blocks x "
+                                                    "this time, an extrapolation (linears only: no attention, norms, head or loss)"},
     }
 
 
