@@ -6,9 +6,11 @@ from .float8 import (  # noqa: F401
     clear_cast_memos,
     config,
     convert_linears_to_fp8,
+    get_scale_rule,
     matmul,
     named_replace,
     scale,
+    set_scale_rule,
 )
 
 __all__ = [
@@ -18,7 +20,9 @@ __all__ = [
     "clear_cast_memos",
     "config",
     "convert_linears_to_fp8",
+    "get_scale_rule",
     "matmul",
     "named_replace",
     "scale",
+    "set_scale_rule",
 ]

@@ -20,6 +20,8 @@ SIGNATURES = {
     "l8_version": [],
     "l8_last_error": [],
     "l8_device_check": [_int],
+    "l8_set_scale_rule": [_int],
+    "l8_get_scale_rule": [],
     "l8_cast_rowwise": [_p, _i64, _i64, _i64, _p, _i64, _p, _p, _p, _p, _i64, _p],
     "l8_cast_rowwise_workspace": [_i64, _i64],
     "l8_cast_rowwise_noalloc": [_p, _i64, _i64, _i64, _p, _i64, _p, _p, _p, _p],

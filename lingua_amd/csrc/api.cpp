@@ -4,6 +4,8 @@
 #include <stdio.h>
 #include <string.h>
 
+#include <atomic>
+
 #include "l8_common.h"
 
 namespace l8 {
@@ -17,6 +19,9 @@ int fail(int code, const char *fmt, ...) {
   va_end(ap);
   return code;
 }
+
+static std::atomic<int> g_scale_rule{L8_SCALE_RULE_DIVIDE};
+int scale_rule() { return g_scale_rule.load(std::memory_order_relaxed); }
 
 static int g_cus[kMaxDev];  // 0 = not queried yet; benign race: every thread writes the same value
 
@@ -41,6 +46,15 @@ int num_cus() {
 extern "C" int l8_version(void) { return 1; }
 
 extern "C" const char *l8_last_error(void) { return l8::g_err; }
+
+extern "C" int l8_set_scale_rule(int rule) {
+  if (rule != L8_SCALE_RULE_DIVIDE && rule != L8_SCALE_RULE_TIMES_INVERSE)
+    return l8::fail(L8_EINVAL, "l8_set_scale_rule: unknown rule %d", rule);
+  l8::g_scale_rule.store(rule, std::memory_order_relaxed);
+  return L8_OK;
+}
+
+extern "C" int l8_get_scale_rule(void) { return l8::scale_rule(); }
 
 extern "C" int l8_device_check(int device) {
   hipDeviceProp_t prop;

@@ -36,7 +36,7 @@ L8_DEV void load_row(v4i (&buf)[NCH], const uint16_t *row, int C, int lane) {
 template <int NCH, bool COLMAX>
 __global__ __launch_bounds__(kRowBlock, 2) void cast_rowwise_kernel(
     const uint16_t *__restrict__ x, int64_t R, int C, int64_t ldx, uint8_t *__restrict__ q, int64_t ldq,
-    float *__restrict__ scale, uint16_t *__restrict__ amax_out, uint16_t *__restrict__ col_partials) {
+    float *__restrict__ scale, uint16_t *__restrict__ amax_out, uint16_t *__restrict__ col_partials, int scale_rule) {
   extern __shared__ uint32_t lds_colmax[];  // [C/2] packed bf16 pairs when COLMAX
   // the next row is prefetched into a second register set unless that would
   // push the wave beyond 256 VGPRs (two waves per SIMD are worth more)
@@ -73,7 +73,7 @@ __global__ __launch_bounds__(kRowBlock, 2) void cast_rowwise_kernel(
     const bool finite = amax_bits < 0x7f80u;
     float s;
     if (finite) {
-      s = scale_from_amax(bf16_bits_to_f32(amax_bits));
+      s = scale_from_amax(bf16_bits_to_f32(amax_bits), scale_rule);
     } else if (amax_bits == 0x7f80u) {
       s = __uint_as_float(0x7f800000u);  // inf / 448
     } else {
@@ -146,7 +146,7 @@ __global__ __launch_bounds__(kRowBlock, 2) void cast_rowwise_kernel(
 template <int NCHW, bool COLMAX>
 __global__ __launch_bounds__(kRowBlock, (NCHW <= 4 ? 4 : (NCHW <= 8 ? 2 : 1))) void cast_rowwise_wg_kernel(
     const uint16_t *__restrict__ x, int64_t R, int C, int64_t ldx, uint8_t *__restrict__ q, int64_t ldq,
-    float *__restrict__ scale, uint16_t *__restrict__ amax_out, uint16_t *__restrict__ col_partials) {
+    float *__restrict__ scale, uint16_t *__restrict__ amax_out, uint16_t *__restrict__ col_partials, int scale_rule) {
   __shared__ uint32_t red[2][kRowWaves];
   const int lane = threadIdx.x & 63;
   const int wave = threadIdx.x >> 6;
@@ -186,7 +186,7 @@ __global__ __launch_bounds__(kRowBlock, (NCHW <= 4 ? 4 : (NCHW <= 8 ? 2 : 1))) v
     for (int w = 0; w < kRowWaves; ++w) amax_bits = max(amax_bits, red[it & 1][w]);
     const bool finite = amax_bits < 0x7f80u;
     float s;
-    if (finite) s = scale_from_amax(bf16_bits_to_f32(amax_bits));
+    if (finite) s = scale_from_amax(bf16_bits_to_f32(amax_bits), scale_rule);
     else s = __uint_as_float(amax_bits == 0x7f80u ? 0x7f800000u : 0x7fc00000u);
     const float recip = recip_exact(s);
     if (threadIdx.x == 0) {
@@ -279,7 +279,7 @@ __global__ __launch_bounds__(256) void zero_u32_kernel(uint32_t *__restrict__ p,
 // one workgroup (the second pass hits L2).
 __global__ __launch_bounds__(kRowBlock) void cast_rowwise_long_kernel(
     const uint16_t *__restrict__ x, int64_t R, int C, int64_t ldx, uint8_t *__restrict__ q, int64_t ldq,
-    float *__restrict__ scale, uint16_t *__restrict__ amax_out, uint32_t *__restrict__ col_amax) {
+    float *__restrict__ scale, uint16_t *__restrict__ amax_out, uint32_t *__restrict__ col_amax, int scale_rule) {
   __shared__ uint32_t red[kRowWaves];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   for (int64_t r = blockIdx.x; r < R; r += gridDim.x) {
@@ -305,7 +305,7 @@ __global__ __launch_bounds__(kRowBlock) void cast_rowwise_long_kernel(
 #pragma unroll
     for (int w = 0; w < kRowWaves; ++w) amax_bits = max(amax_bits, red[w]);
     float s;
-    if (amax_bits < 0x7f80u) s = scale_from_amax(bf16_bits_to_f32(amax_bits));
+    if (amax_bits < 0x7f80u) s = scale_from_amax(bf16_bits_to_f32(amax_bits), scale_rule);
     else s = __uint_as_float(amax_bits == 0x7f80u ? 0x7f800000u : 0x7fc00000u);
     const float recip = recip_exact(s);
     if (threadIdx.x == 0) {
@@ -364,33 +364,33 @@ __global__ __launch_bounds__(1024) void amax_reduce_kernel(const uint16_t *__res
 // ---------------------------------------------------------------------------
 // Tensor-wise, same layout out as in: pure streaming.
 // ---------------------------------------------------------------------------
-L8_DEV float scale_from_amax_bits16(uint32_t amax_bits) {
-  if (amax_bits < 0x7f80u) return scale_from_amax(bf16_bits_to_f32(amax_bits));
+L8_DEV float scale_from_amax_bits16(uint32_t amax_bits, int scale_rule) {
+  if (amax_bits < 0x7f80u) return scale_from_amax(bf16_bits_to_f32(amax_bits), scale_rule);
   return __uint_as_float(amax_bits == 0x7f80u ? 0x7f800000u : 0x7fc00000u);
 }
-L8_DEV float scale_from_amax_bits32(uint32_t amax_bits) {  // fp32 bit pattern of a non-negative amax
-  if (amax_bits < 0x7f800000u) return scale_from_amax(__uint_as_float(amax_bits));
+L8_DEV float scale_from_amax_bits32(uint32_t amax_bits, int scale_rule) {  // fp32 bit pattern of a non-negative amax
+  if (amax_bits < 0x7f800000u) return scale_from_amax(__uint_as_float(amax_bits), scale_rule);
   return __uint_as_float(amax_bits == 0x7f800000u ? 0x7f800000u : 0x7fc00000u);
 }
 
 // A device-resident amax scalar, bf16 or fp32 (sign ignored): its scale, and whether it is finite.
-L8_DEV float scale_from_amax_scalar(const void *amax, int amax_f32, bool &finite) {
+L8_DEV float scale_from_amax_scalar(const void *amax, int amax_f32, bool &finite, int scale_rule) {
   if (amax_f32) {
     const uint32_t bits = *(const uint32_t *)amax & 0x7fffffffu;
     finite = bits < 0x7f800000u;
-    return scale_from_amax_bits32(bits);
+    return scale_from_amax_bits32(bits, scale_rule);
   }
   const uint32_t bits = *(const uint16_t *)amax & 0x7fffu;
   finite = bits < 0x7f80u;
-  return scale_from_amax_bits16(bits);
+  return scale_from_amax_bits16(bits, scale_rule);
 }
 
 __global__ __launch_bounds__(256) void cast_tensorwise_kernel(const uint16_t *__restrict__ x, int64_t R, int C,
                                                               int64_t ldx, const void *__restrict__ amax, int amax_f32,
                                                               uint8_t *__restrict__ q, int64_t ldq,
-                                                              float *__restrict__ scale) {
+                                                              float *__restrict__ scale, int scale_rule) {
   bool finite;
-  const float s = scale_from_amax_scalar(amax, amax_f32, finite);
+  const float s = scale_from_amax_scalar(amax, amax_f32, finite, scale_rule);
   const float recip = recip_exact(s);
   if (blockIdx.x == 0 && threadIdx.x == 0) scale[0] = s;
   const int cpr = C / 8;  // 16-byte chunks per row
@@ -413,14 +413,14 @@ __global__ __launch_bounds__(256) void cast_tensorwise_kernel(const uint16_t *__
 __global__ __launch_bounds__(256) void cast_rowwise_given_amax_kernel(const uint16_t *__restrict__ x, int64_t R, int C,
                                                                       int64_t ldx, const void *__restrict__ amax, int amax_f32,
                                                                       uint8_t *__restrict__ q, int64_t ldq,
-                                                                      float *__restrict__ scale) {
+                                                                      float *__restrict__ scale, int scale_rule) {
   const int cpr = C / 8;  // 16-byte chunks per row
   const int64_t total = R * cpr;
   for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < total; i += (int64_t)gridDim.x * 256) {
     const int64_t r = i / cpr;
     const int c = (int)(i - r * cpr) * 8;
     // clamp(min=EPS) also lifts a negative amax
-    const float s = scale_from_amax(amax_f32 ? ((const float *)amax)[r] : bf16_bits_to_f32(((const uint16_t *)amax)[r]));
+    const float s = scale_from_amax(amax_f32 ? ((const float *)amax)[r] : bf16_bits_to_f32(((const uint16_t *)amax)[r]), scale_rule);
     const float recip = recip_exact(s);
     if (c == 0) scale[r] = s;
     const v4i v = __builtin_nontemporal_load((const v4i *)(x + r * ldx + c));
@@ -459,7 +459,7 @@ template <bool PER_COL>
 __global__ __launch_bounds__(256) void cast_transposed_kernel(
     const uint16_t *__restrict__ x, int64_t R, int C, int64_t ldx, const void *__restrict__ amax_scalar, int amax_f32,
     const uint32_t *__restrict__ col_amax, uint8_t *__restrict__ q, int64_t ldq, float *__restrict__ scale,
-    int vec_store) {
+    int vec_store, int scale_rule) {
   __shared__ __attribute__((aligned(16))) uint8_t tile[kTC * kTStride];
   __shared__ float recips[kTC];
   const int t = threadIdx.x;
@@ -498,7 +498,7 @@ __global__ __launch_bounds__(256) void cast_transposed_kernel(
       float rc = 0.0f;
       if (col < C) {
         const uint32_t bits = col_amax[col];
-        const float s = scale_from_amax_bits32(bits);
+        const float s = scale_from_amax_bits32(bits, scale_rule);
         rc = recip_exact(s);
         if (bits >= 0x7f800000u) rc = __uint_as_float(0x7fc00000u);  // flag: slow path for this column
         if (rt == 0) scale[col] = s;
@@ -512,7 +512,7 @@ __global__ __launch_bounds__(256) void cast_transposed_kernel(
 #pragma unroll
     for (int j = 0; j < 8; ++j) rcp[j] = recips[cc * 8 + j];
   } else {
-    const float s = scale_from_amax_scalar(amax_scalar, amax_f32, finite);
+    const float s = scale_from_amax_scalar(amax_scalar, amax_f32, finite, scale_rule);
     const float rc = recip_exact(s);
 #pragma unroll
     for (int j = 0; j < 8; ++j) rcp[j] = rc;
@@ -542,7 +542,7 @@ __global__ __launch_bounds__(256) void cast_transposed_kernel(
         float rc = rcp[j];
         if (PER_COL) {
           const uint32_t bits = col_amax[c + j < C ? c + j : 0];
-          rc = recip_exact(scale_from_amax_bits32(bits));
+          rc = recip_exact(scale_from_amax_bits32(bits, scale_rule));
         }
         packed = 0;
 #pragma unroll
@@ -618,12 +618,12 @@ static int launch_rowwise(const void *x, int64_t R, int64_t C, int64_t ldx, void
   if (col_amax) {
     const size_t lds = (size_t)C * sizeof(uint16_t);
     hipLaunchKernelGGL((cast_rowwise_kernel<NCH, true>), dim3((unsigned)blocks), dim3(kRowBlock), lds, st,
-                       (const uint16_t *)x, R, (int)C, ldx, (uint8_t *)q, ldq, scale, (uint16_t *)amax, (uint16_t *)ws);
+                       (const uint16_t *)x, R, (int)C, ldx, (uint8_t *)q, ldq, scale, (uint16_t *)amax, (uint16_t *)ws, l8::scale_rule());
     L8_HIP(hipGetLastError());
     return fold_colmax(ws, blocks, C, col_amax, st);
   }
   hipLaunchKernelGGL((cast_rowwise_kernel<NCH, false>), dim3((unsigned)blocks), dim3(kRowBlock), 0, st,
-                     (const uint16_t *)x, R, (int)C, ldx, (uint8_t *)q, ldq, scale, (uint16_t *)amax, (uint16_t *)nullptr);
+                     (const uint16_t *)x, R, (int)C, ldx, (uint8_t *)q, ldq, scale, (uint16_t *)amax, (uint16_t *)nullptr, l8::scale_rule());
   L8_HIP(hipGetLastError());
   return L8_OK;
 }
@@ -634,12 +634,12 @@ static int launch_rowwise_wg(const void *x, int64_t R, int64_t C, int64_t ldx, v
   const int64_t blocks = rowwise_blocks(R, C, col_amax != nullptr);
   if (col_amax) {
     hipLaunchKernelGGL((cast_rowwise_wg_kernel<NCHW, true>), dim3((unsigned)blocks), dim3(kRowBlock), 0, st,
-                       (const uint16_t *)x, R, (int)C, ldx, (uint8_t *)q, ldq, scale, (uint16_t *)amax, (uint16_t *)ws);
+                       (const uint16_t *)x, R, (int)C, ldx, (uint8_t *)q, ldq, scale, (uint16_t *)amax, (uint16_t *)ws, l8::scale_rule());
     L8_HIP(hipGetLastError());
     return fold_colmax(ws, blocks, C, col_amax, st);
   }
   hipLaunchKernelGGL((cast_rowwise_wg_kernel<NCHW, false>), dim3((unsigned)blocks), dim3(kRowBlock), 0, st,
-                     (const uint16_t *)x, R, (int)C, ldx, (uint8_t *)q, ldq, scale, (uint16_t *)amax, (uint16_t *)nullptr);
+                     (const uint16_t *)x, R, (int)C, ldx, (uint8_t *)q, ldq, scale, (uint16_t *)amax, (uint16_t *)nullptr, l8::scale_rule());
   L8_HIP(hipGetLastError());
   return L8_OK;
 }
@@ -682,7 +682,7 @@ static int cast_rowwise_impl(const char *what, const void *x, int64_t R, int64_t
     if (rc != L8_OK) return rc;
   }
   hipLaunchKernelGGL(cast_rowwise_long_kernel, dim3((unsigned)blocks), dim3(kRowBlock), 0, st, (const uint16_t *)x, R,
-                     (int)C, ldx, (uint8_t *)q, ldq, scale, (uint16_t *)amax, (uint32_t *)col_amax);
+                     (int)C, ldx, (uint8_t *)q, ldq, scale, (uint16_t *)amax, (uint32_t *)col_amax, l8::scale_rule());
   L8_HIP(hipGetLastError());
   return L8_OK;
 }
@@ -769,7 +769,7 @@ extern "C" int l8_cast_rowwise_given_amax(const void *x, int64_t R, int64_t C, i
   const int64_t cap = (int64_t)num_cus() * 16;
   if (blocks > cap) blocks = cap;
   hipLaunchKernelGGL(cast_rowwise_given_amax_kernel, dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream,
-                     (const uint16_t *)x, R, (int)C, ldx, amax, amax_dtype, (uint8_t *)q, ldq, scale);
+                     (const uint16_t *)x, R, (int)C, ldx, amax, amax_dtype, (uint8_t *)q, ldq, scale, l8::scale_rule());
   L8_HIP(hipGetLastError());
   return L8_OK;
 }
@@ -812,11 +812,11 @@ static int launch_transposed(bool per_col, const void *x, int64_t R, int64_t C, 
   if (per_col)
     hipLaunchKernelGGL((cast_transposed_kernel<true>), dim3((unsigned)gx, (unsigned)gy), dim3(256), 0, st,
                        (const uint16_t *)x, R, (int)C, ldx, (const void *)nullptr, 0, (const uint32_t *)col_amax,
-                       (uint8_t *)q, ldq, scale, vec);
+                       (uint8_t *)q, ldq, scale, vec, l8::scale_rule());
   else
     hipLaunchKernelGGL((cast_transposed_kernel<false>), dim3((unsigned)gx, (unsigned)gy), dim3(256), 0, st,
                        (const uint16_t *)x, R, (int)C, ldx, amax, amax_f32, (const uint32_t *)nullptr,
-                       (uint8_t *)q, ldq, scale, vec);
+                       (uint8_t *)q, ldq, scale, vec, l8::scale_rule());
   L8_HIP(hipGetLastError());
   return L8_OK;
 }
@@ -842,7 +842,7 @@ extern "C" int l8_cast_tensorwise(const void *x, int64_t R, int64_t C, int64_t l
   const int64_t cap = (int64_t)num_cus() * 16;
   if (blocks > cap) blocks = cap;
   hipLaunchKernelGGL(cast_tensorwise_kernel, dim3((unsigned)blocks), dim3(256), 0, st, (const uint16_t *)x, R, (int)C,
-                     ldx, amax, amax_dtype, (uint8_t *)q, ldq, scale);
+                     ldx, amax, amax_dtype, (uint8_t *)q, ldq, scale, l8::scale_rule());
   L8_HIP(hipGetLastError());
   return L8_OK;
 }

@@ -27,6 +27,9 @@ int fail(int code, const char *fmt, ...);  // records the thread-local message, 
 
 int num_cus();  // compute units of the current device (cached per device)
 
+// How every cast evaluates clamp(amax, EPS) / 448 (l8_set_scale_rule); read once per launch and handed to the kernel.
+int scale_rule();
+
 // Per-device one-time set-up (function attributes are per device): index of the
 // current device into tables of kMaxDev entries, or -1 (then nothing is cached).
 constexpr int kMaxDev = 64;
@@ -48,11 +51,14 @@ constexpr float kE4M3Max = 448.0f;   // torch.finfo(float8_e4m3fn).max
 
 L8_DEV float bf16_bits_to_f32(uint32_t h) { return __uint_as_float(h << 16); }
 
-// scale = clamp(f32(amax), min=EPS) / 448 with a correctly rounded division
-// (lingua/float8.py:44-45).  NaN passes through the clamp, as torch.clamp does.
-L8_DEV float scale_from_amax(float amax) {
+// scale = clamp(f32(amax), min=EPS) / 448 (lingua/float8.py:44-45).  NaN passes through the clamp, as torch.clamp
+// does.  Rule L8_SCALE_RULE_DIVIDE is the correctly rounded division, which is what the ATen CPU kernel computes;
+// rule L8_SCALE_RULE_TIMES_INVERSE is what the ATen GPU kernel computes for a division by a Python scalar: the product
+// with fp32(1/448), which differs from the quotient in the last bit for about half of all amaxes.
+constexpr float kInvE4M3Max = 1.0f / 448.0f;
+L8_DEV float scale_from_amax(float amax, int scale_rule) {
   float a = (amax < kEps) ? kEps : amax;
-  return a / kE4M3Max;
+  return scale_rule == L8_SCALE_RULE_TIMES_INVERSE ? a * kInvE4M3Max : a / kE4M3Max;
 }
 L8_DEV float recip_exact(float s) { return 1.0f / s; }
 
@@ -154,10 +160,10 @@ struct RowScale {
   float s, recip;
   bool finite;
 };
-L8_DEV RowScale row_scale(uint32_t amax_bits) {
+L8_DEV RowScale row_scale(uint32_t amax_bits, int scale_rule) {
   RowScale r;
   r.finite = amax_bits < 0x7f80u;
-  r.s = r.finite ? scale_from_amax(bf16_bits_to_f32(amax_bits))
+  r.s = r.finite ? scale_from_amax(bf16_bits_to_f32(amax_bits), scale_rule)
                  : __uint_as_float(amax_bits == 0x7f80u ? 0x7f800000u : 0x7fc00000u);
   r.recip = recip_exact(r.s);
   return r;

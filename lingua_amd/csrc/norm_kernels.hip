@@ -42,7 +42,7 @@ template <int NCHW, bool COLMAX, bool W_F32>
 __global__ __launch_bounds__(kNormBlock, 2) void rmsnorm_cast_rowwise_kernel(
     const uint16_t *__restrict__ x, const void *__restrict__ w, int64_t R, int C, int64_t ldx, float eps,
     uint16_t *__restrict__ y, int64_t ldy, uint8_t *__restrict__ q, int64_t ldq, float *__restrict__ scale,
-    float *__restrict__ rstd, uint16_t *__restrict__ col_partials) {
+    float *__restrict__ rstd, uint16_t *__restrict__ col_partials, int scale_rule) {
   __shared__ float red_ss[2][kNormWaves];
   __shared__ uint32_t red_mx[2][kNormWaves];
   extern __shared__ __attribute__((aligned(16))) uint8_t dyn_lds[];
@@ -128,7 +128,7 @@ __global__ __launch_bounds__(kNormBlock, 2) void rmsnorm_cast_rowwise_kernel(
     uint32_t amax_bits = 0;
 #pragma unroll
     for (int wv = 0; wv < kNormWaves; ++wv) amax_bits = max(amax_bits, red_mx[it & 1][wv]);
-    const RowScale rs = row_scale(amax_bits);
+    const RowScale rs = row_scale(amax_bits, scale_rule);
     if (threadIdx.x == 0 && scale) scale[r] = rs.s;
     if (q) {
       uint8_t *qrow = q + r * ldq;
@@ -276,13 +276,13 @@ static int launch_norm(const void *x, const void *w, int64_t R, int64_t C, int64
     const size_t lds = colmax_in_lds<NCHW, 1>() ? (size_t)C * 2 : 0;
     hipLaunchKernelGGL((rmsnorm_cast_rowwise_kernel<NCHW, true, W_F32>), dim3((unsigned)blocks), dim3(kNormBlock), lds, st,
                        (const uint16_t *)x, w, R, (int)C, ldx, eps, (uint16_t *)y, ldy, (uint8_t *)q, ldq, scale, rstd,
-                       (uint16_t *)ws);
+                       (uint16_t *)ws, l8::scale_rule());
     L8_HIP(hipGetLastError());
     return fold_colmax(ws, blocks, C, col_amax, st);
   }
   hipLaunchKernelGGL((rmsnorm_cast_rowwise_kernel<NCHW, false, W_F32>), dim3((unsigned)blocks), dim3(kNormBlock), 0, st,
                      (const uint16_t *)x, w, R, (int)C, ldx, eps, (uint16_t *)y, ldy, (uint8_t *)q, ldq, scale, rstd,
-                     (uint16_t *)nullptr);
+                     (uint16_t *)nullptr, l8::scale_rule());
   L8_HIP(hipGetLastError());
   return L8_OK;
 }

@@ -70,7 +70,7 @@ template <int NCHW, bool COLMAX>
 __global__ __launch_bounds__(kGateBlock, 2) void swiglu_cast_rowwise_kernel(
     const uint16_t *__restrict__ h1, const uint16_t *__restrict__ h3, int64_t R, int C, int64_t ld1, int64_t ld3,
     uint16_t *__restrict__ hout, int64_t ldh, uint8_t *__restrict__ q, int64_t ldq, float *__restrict__ scale,
-    uint16_t *__restrict__ amax_out, uint16_t *__restrict__ col_partials) {
+    uint16_t *__restrict__ amax_out, uint16_t *__restrict__ col_partials, int scale_rule) {
   __shared__ uint32_t red[2][kGateWaves];
   extern __shared__ __attribute__((aligned(16))) uint8_t dyn_lds[];
   constexpr bool CLDS = COLMAX && colmax_in_lds<NCHW, 1>();
@@ -128,7 +128,7 @@ __global__ __launch_bounds__(kGateBlock, 2) void swiglu_cast_rowwise_kernel(
     uint32_t amax_bits = 0;
 #pragma unroll
     for (int w = 0; w < kGateWaves; ++w) amax_bits = max(amax_bits, red[it & 1][w]);
-    const RowScale rs = row_scale(amax_bits);
+    const RowScale rs = row_scale(amax_bits, scale_rule);
     if (threadIdx.x == 0) {
       if (scale) scale[r] = rs.s;
       if (amax_out) amax_out[r] = (uint16_t)amax_bits;
@@ -161,7 +161,7 @@ __global__ __launch_bounds__(kGateBlock, 2) void swiglu_bwd_cast_rowwise_kernel(
     const uint16_t *__restrict__ dh, const uint16_t *__restrict__ h1, const uint16_t *__restrict__ h3, int64_t R, int C,
     int64_t lddh, int64_t ld1, int64_t ld3, uint16_t *__restrict__ g1out, uint16_t *__restrict__ g3out, int64_t ldg,
     uint8_t *__restrict__ q1, uint8_t *__restrict__ q3, int64_t ldq, float *__restrict__ scale1,
-    float *__restrict__ scale3, uint16_t *__restrict__ col_partials1, uint16_t *__restrict__ col_partials3) {
+    float *__restrict__ scale3, uint16_t *__restrict__ col_partials1, uint16_t *__restrict__ col_partials3, int scale_rule) {
   __shared__ uint32_t red[2][2][kGateWaves];
   extern __shared__ __attribute__((aligned(16))) uint8_t dyn_lds[];
   constexpr bool CLDS = COLMAX && colmax_in_lds<NCHW, 2>();
@@ -235,7 +235,7 @@ __global__ __launch_bounds__(kGateBlock, 2) void swiglu_bwd_cast_rowwise_kernel(
       bits1 = max(bits1, red[it & 1][0][w]);
       bits3 = max(bits3, red[it & 1][1][w]);
     }
-    const RowScale rs1 = row_scale(bits1), rs3 = row_scale(bits3);
+    const RowScale rs1 = row_scale(bits1, scale_rule), rs3 = row_scale(bits3, scale_rule);
     if (threadIdx.x == 0) {
       scale1[r] = rs1.s;
       scale3[r] = rs3.s;
@@ -279,7 +279,7 @@ template <bool COLMAX>
 __global__ __launch_bounds__(kWideBlock) void swiglu_cast_rowwise_wide_kernel(
     const uint16_t *__restrict__ h1, const uint16_t *__restrict__ h3, int64_t R, int C, int64_t ld1, int64_t ld3,
     uint16_t *__restrict__ hout, int64_t ldh, uint8_t *__restrict__ q, int64_t ldq, float *__restrict__ scale,
-    uint16_t *__restrict__ amax_out, uint16_t *__restrict__ col_partials) {
+    uint16_t *__restrict__ amax_out, uint16_t *__restrict__ col_partials, int scale_rule) {
   __shared__ uint32_t red[2][kWideWaves];
   extern __shared__ __attribute__((aligned(16))) uint8_t dyn_lds[];
   v4i *lds_cm = (v4i *)dyn_lds;  // [C / 8]
@@ -313,7 +313,7 @@ __global__ __launch_bounds__(kWideBlock) void swiglu_cast_rowwise_wide_kernel(
     uint32_t amax_bits = 0;
 #pragma unroll
     for (int w = 0; w < kWideWaves; ++w) amax_bits = max(amax_bits, red[it & 1][w]);
-    const RowScale rs = row_scale(amax_bits);
+    const RowScale rs = row_scale(amax_bits, scale_rule);
     if (threadIdx.x == 0) {
       if (scale) scale[r] = rs.s;
       if (amax_out) amax_out[r] = (uint16_t)amax_bits;
@@ -345,7 +345,7 @@ __global__ __launch_bounds__(kWideBlock) void swiglu_bwd_cast_rowwise_wide_kerne
     const uint16_t *__restrict__ dh, const uint16_t *__restrict__ h1, const uint16_t *__restrict__ h3, int64_t R, int C,
     int64_t lddh, int64_t ld1, int64_t ld3, uint16_t *__restrict__ g1out, uint16_t *__restrict__ g3out, int64_t ldg,
     uint8_t *__restrict__ q1, uint8_t *__restrict__ q3, int64_t ldq, float *__restrict__ scale1,
-    float *__restrict__ scale3, uint16_t *__restrict__ col_partials1, uint16_t *__restrict__ col_partials3) {
+    float *__restrict__ scale3, uint16_t *__restrict__ col_partials1, uint16_t *__restrict__ col_partials3, int scale_rule) {
   __shared__ uint32_t red[2][2][kWideWaves];
   extern __shared__ __attribute__((aligned(16))) uint8_t dyn_lds[];
   v4i *lds_cm1 = (v4i *)dyn_lds, *lds_cm3 = lds_cm1 + C / 8;  // [C / 8] each
@@ -396,7 +396,7 @@ __global__ __launch_bounds__(kWideBlock) void swiglu_bwd_cast_rowwise_wide_kerne
       bits1 = max(bits1, red[it & 1][0][w]);
       bits3 = max(bits3, red[it & 1][1][w]);
     }
-    const RowScale rs1 = row_scale(bits1), rs3 = row_scale(bits3);
+    const RowScale rs1 = row_scale(bits1, scale_rule), rs3 = row_scale(bits3, scale_rule);
     if (threadIdx.x == 0) {
       scale1[r] = rs1.s;
       scale3[r] = rs3.s;
@@ -450,13 +450,13 @@ static int launch_fwd_wide(const void *h1, const void *h3, int64_t R, int64_t C,
     if (rc != L8_OK) return rc;
     hipLaunchKernelGGL((swiglu_cast_rowwise_wide_kernel<true>), dim3((unsigned)blocks), dim3(kWideBlock), lds, st,
                        (const uint16_t *)h1, (const uint16_t *)h3, R, (int)C, ld1, ld3, (uint16_t *)h, ldh, (uint8_t *)q, ldq,
-                       scale, (uint16_t *)amax, (uint16_t *)ws);
+                       scale, (uint16_t *)amax, (uint16_t *)ws, l8::scale_rule());
     L8_HIP(hipGetLastError());
     return fold_colmax(ws, blocks, C, col_amax, st);
   }
   hipLaunchKernelGGL((swiglu_cast_rowwise_wide_kernel<false>), dim3((unsigned)blocks), dim3(kWideBlock), 0, st,
                      (const uint16_t *)h1, (const uint16_t *)h3, R, (int)C, ld1, ld3, (uint16_t *)h, ldh, (uint8_t *)q, ldq,
-                     scale, (uint16_t *)amax, (uint16_t *)nullptr);
+                     scale, (uint16_t *)amax, (uint16_t *)nullptr, l8::scale_rule());
   L8_HIP(hipGetLastError());
   return L8_OK;
 }
@@ -473,7 +473,7 @@ static int launch_bwd_wide(const void *dh, const void *h1, const void *h3, int64
     if (rc != L8_OK) return rc;
     hipLaunchKernelGGL((swiglu_bwd_cast_rowwise_wide_kernel<true>), dim3((unsigned)blocks), dim3(kWideBlock), lds, st,
                        (const uint16_t *)dh, (const uint16_t *)h1, (const uint16_t *)h3, R, (int)C, lddh, ld1, ld3,
-                       (uint16_t *)g1, (uint16_t *)g3, ldg, (uint8_t *)q1, (uint8_t *)q3, ldq, s1, s3, w1, w3);
+                       (uint16_t *)g1, (uint16_t *)g3, ldg, (uint8_t *)q1, (uint8_t *)q3, ldq, s1, s3, w1, w3, l8::scale_rule());
     L8_HIP(hipGetLastError());
     rc = fold_colmax(w1, blocks, C, ca1, st);
     if (rc != L8_OK) return rc;
@@ -482,7 +482,7 @@ static int launch_bwd_wide(const void *dh, const void *h1, const void *h3, int64
   hipLaunchKernelGGL((swiglu_bwd_cast_rowwise_wide_kernel<false>), dim3((unsigned)blocks), dim3(kWideBlock), 0, st,
                      (const uint16_t *)dh, (const uint16_t *)h1, (const uint16_t *)h3, R, (int)C, lddh, ld1, ld3,
                      (uint16_t *)g1, (uint16_t *)g3, ldg, (uint8_t *)q1, (uint8_t *)q3, ldq, s1, s3, (uint16_t *)nullptr,
-                     (uint16_t *)nullptr);
+                     (uint16_t *)nullptr, l8::scale_rule());
   L8_HIP(hipGetLastError());
   return L8_OK;
 }
@@ -502,13 +502,13 @@ static int launch_fwd(const void *h1, const void *h3, int64_t R, int64_t C, int6
     }
     hipLaunchKernelGGL((swiglu_cast_rowwise_kernel<NCHW, true>), dim3((unsigned)blocks), dim3(kGateBlock), lds, st,
                        (const uint16_t *)h1, (const uint16_t *)h3, R, (int)C, ld1, ld3, (uint16_t *)h, ldh, (uint8_t *)q, ldq,
-                       scale, (uint16_t *)amax, (uint16_t *)ws);
+                       scale, (uint16_t *)amax, (uint16_t *)ws, l8::scale_rule());
     L8_HIP(hipGetLastError());
     return fold_colmax(ws, blocks, C, col_amax, st);
   }
   hipLaunchKernelGGL((swiglu_cast_rowwise_kernel<NCHW, false>), dim3((unsigned)blocks), dim3(kGateBlock), 0, st,
                      (const uint16_t *)h1, (const uint16_t *)h3, R, (int)C, ld1, ld3, (uint16_t *)h, ldh, (uint8_t *)q, ldq,
-                     scale, (uint16_t *)amax, (uint16_t *)nullptr);
+                     scale, (uint16_t *)amax, (uint16_t *)nullptr, l8::scale_rule());
   L8_HIP(hipGetLastError());
   return L8_OK;
 }
@@ -530,7 +530,7 @@ static int launch_bwd(const void *dh, const void *h1, const void *h3, int64_t R,
     }
     hipLaunchKernelGGL((swiglu_bwd_cast_rowwise_kernel<NCHW, true>), dim3((unsigned)blocks), dim3(kGateBlock), lds, st,
                        (const uint16_t *)dh, (const uint16_t *)h1, (const uint16_t *)h3, R, (int)C, lddh, ld1, ld3,
-                       (uint16_t *)g1, (uint16_t *)g3, ldg, (uint8_t *)q1, (uint8_t *)q3, ldq, s1, s3, w1, w3);
+                       (uint16_t *)g1, (uint16_t *)g3, ldg, (uint8_t *)q1, (uint8_t *)q3, ldq, s1, s3, w1, w3, l8::scale_rule());
     L8_HIP(hipGetLastError());
     const int rc = fold_colmax(w1, blocks, C, ca1, st);
     if (rc != L8_OK) return rc;
@@ -539,7 +539,7 @@ static int launch_bwd(const void *dh, const void *h1, const void *h3, int64_t R,
   hipLaunchKernelGGL((swiglu_bwd_cast_rowwise_kernel<NCHW, false>), dim3((unsigned)blocks), dim3(kGateBlock), 0, st,
                      (const uint16_t *)dh, (const uint16_t *)h1, (const uint16_t *)h3, R, (int)C, lddh, ld1, ld3,
                      (uint16_t *)g1, (uint16_t *)g3, ldg, (uint8_t *)q1, (uint8_t *)q3, ldq, s1, s3, (uint16_t *)nullptr,
-                     (uint16_t *)nullptr);
+                     (uint16_t *)nullptr, l8::scale_rule());
   L8_HIP(hipGetLastError());
   return L8_OK;
 }

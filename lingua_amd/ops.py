@@ -303,6 +303,24 @@ def gemm_pick(M: int, N: int, K: int) -> Tuple[int, str]:
     return algo, lib.l8_gemm_algo_name(algo).decode()
 
 
+SCALE_RULES = {"divide": 0, "times_inverse": 1}
+
+
+def set_scale_rule(rule: str) -> None:
+    """How the casts evaluate ``clamp(amax, EPS) / 448`` (lingua/float8.py:44): ``"divide"`` (default) is the correctly
+    rounded fp32 quotient, what ATen's CPU kernel computes; ``"times_inverse"`` is amax * fp32(1/448), what ATen's GPU
+    kernel computes for a division by a Python scalar, i.e. the reference's scales when it runs on a GPU.  Process-wide;
+    applies to casts launched after the call."""
+    if rule not in SCALE_RULES:
+        raise RuntimeError(f"unknown scale rule {rule!r}; known: {sorted(SCALE_RULES)}")
+    _lib.check(_lib.load().l8_set_scale_rule(SCALE_RULES[rule]), "l8_set_scale_rule")
+
+
+def get_scale_rule() -> str:
+    code = _lib.load().l8_get_scale_rule()
+    return next(name for name, c in SCALE_RULES.items() if c == code)
+
+
 def gemm_algos() -> Tuple[str, ...]:
     lib = _lib.load()
     return tuple(lib.l8_gemm_algo_name(i + 1).decode() for i in range(lib.l8_gemm_algo_count()))

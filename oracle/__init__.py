@@ -58,12 +58,38 @@ def lib():
         L.l8o_col_sum.argtypes = [_p, _i64, _i64, _i64, _p]
         L.l8o_e4m3fn_from_f32_array.argtypes = [_p, _i64, _p]
         L.l8o_scale_from_amax_array.argtypes = [_p, _i64, _p]
+        L.l8o_set_scale_rule.argtypes = [ctypes.c_int]
+        L.l8o_set_scale_rule.restype = None
+        L.l8o_get_scale_rule.restype = ctypes.c_int
         for name in ("l8o_row_amax", "l8o_col_amax", "l8o_cast_rowwise", "l8o_cast_tensorwise",
                      "l8o_cast_colwise_transposed", "l8o_gemm_nt", "l8o_gemm_nt_f64", "l8o_col_sum",
                      "l8o_e4m3fn_from_f32_array", "l8o_scale_from_amax_array"):
             getattr(L, name).restype = None
         _lib = L
     return _lib
+
+
+class scale_rule:
+    """``with oracle.scale_rule("times_inverse"):`` -- both restatements evaluate ``clamp(amax) / 448`` the way
+    ATen's GPU kernel does (product with fp32(1/448)) instead of the correctly rounded quotient of ATen's CPU kernel
+    ("divide", the default)."""
+    RULES = {"divide": 0, "times_inverse": 1}
+
+    def __init__(self, rule: str):
+        self.rule = self.RULES[rule]
+
+    def __enter__(self):
+        from . import recipe_torch
+        self.before = lib().l8o_get_scale_rule()
+        lib().l8o_set_scale_rule(self.rule)
+        recipe_torch.SCALE_TIMES_INVERSE = bool(self.rule)
+        return self
+
+    def __exit__(self, *exc):
+        from . import recipe_torch
+        lib().l8o_set_scale_rule(self.before)
+        recipe_torch.SCALE_TIMES_INVERSE = bool(self.before)
+        return False
 
 
 # ----------------------------------------------------------------------------

@@ -12,6 +12,7 @@
  *   - tile-broadcast multiply (row / tensor)  lingua/float8.py:24-30
  *   - scale(t, amax): s = max(f32(amax),EPS)/448 ; q = e4m3fn(t * (1/s))
  *                                             lingua/float8.py:43-47
+ *     (the quotient as ATen's CPU kernel rounds it, or, under l8o_set_scale_rule(1), as ATen's GPU kernel does)
  *   - matmul(): NT product of the two quantised operands, fp32 accumulation,
  *     scales applied to the product, optional bias, bf16 result
  *                                             lingua/float8.py:50-79
@@ -96,11 +97,24 @@ L8O_EXPORT float l8o_e4m3fn_to_f32(uint8_t b) {
 }
 
 /* scale = clamp(f32(amax), min=EPS) / 448  -- lingua/float8.py:44-45.
- * torch.clamp keeps NaN; the division is a correctly rounded fp32 division. */
+ * torch.clamp keeps NaN.  Rule 0 (default): the division is a correctly rounded fp32 division, which is what
+ * ATen's CPU kernel computes.  Rule 1: ATen's GPU kernel divides a tensor by a Python scalar by multiplying with
+ * the scalar's fp32 reciprocal, so the reference run on a GPU computes amax * fp32(1/448); the product differs
+ * from the quotient in the last bit for about half of all amaxes.  (Pinned on the GPU against PyTorch's own
+ * kernel over every bf16 amax, and here against numpy float32 arithmetic.) */
+static int g_scale_rule = 0;
+L8O_EXPORT void l8o_set_scale_rule(int rule) { g_scale_rule = rule; }
+L8O_EXPORT int l8o_get_scale_rule(void) { return g_scale_rule; }
 L8O_EXPORT float l8o_scale_from_amax(uint16_t amax_bf16) {
   volatile float a = bf16_to_f32(amax_bf16);
   const float eps = 1e-12f;
   if (a < eps) a = eps;                       /* false for NaN: NaN passes through */
+  if (g_scale_rule == 1) {
+    volatile float one = 1.0f, max = 448.0f;
+    volatile float inv = one / max;
+    volatile float s = a * inv;
+    return s;
+  }
   volatile float s = a / 448.0f;
   return s;
 }

@@ -13,6 +13,9 @@ import torch
 
 EPS = 1e-12  # lingua/float8.py:11
 E4M3_MAX = torch.finfo(torch.float8_e4m3fn).max  # 448.0
+# ATen's GPU kernel divides a tensor by a Python scalar by multiplying with the scalar's fp32 reciprocal; its CPU
+# kernel divides.  True makes scale() on CPU tensors do what the GPU kernel does (oracle.scale_rule sets this).
+SCALE_TIMES_INVERSE = False
 
 
 def row_amax(t: torch.Tensor) -> torch.Tensor:
@@ -36,7 +39,10 @@ def tile_broadcast(b: torch.Tensor, shape) -> torch.Tensor:
 
 def scale(t: torch.Tensor, amax_t: torch.Tensor):
     """lingua/float8.py:43-47.  amax_t is [R,1] (row-wise), [1,1] (tensor-wise) or [R,g] (g column groups per row)."""
-    scale_t = torch.clamp(amax_t.float(), min=EPS) / E4M3_MAX
+    if SCALE_TIMES_INVERSE and not amax_t.is_cuda:
+        scale_t = torch.clamp(amax_t.float(), min=EPS) * (torch.ones((), dtype=torch.float32) / E4M3_MAX)
+    else:
+        scale_t = torch.clamp(amax_t.float(), min=EPS) / E4M3_MAX
     recip = scale_t.reciprocal()
     t_fp8 = (t * tile_broadcast(recip, t.shape)).to(torch.float8_e4m3fn)
     return t_fp8, scale_t

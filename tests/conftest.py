@@ -25,3 +25,17 @@ def pytest_collection_modifyitems(config, items):
 
 
 from bench_workloads import rel_l2, seeded_bf16  # noqa: E402,F401  (tests import them from here)
+
+
+@pytest.fixture
+def gpu_division_rule():
+    """Library and oracle both evaluate clamp(amax) / 448 the way ATen's GPU kernel does (product with fp32(1/448))
+    for the duration of a test; the default (the correctly rounded quotient) is restored afterwards."""
+    import lingua_amd
+    import oracle
+    lingua_amd.set_scale_rule("times_inverse")
+    try:
+        with oracle.scale_rule("times_inverse"):
+            yield
+    finally:
+        lingua_amd.set_scale_rule("divide")

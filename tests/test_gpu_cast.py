@@ -257,3 +257,57 @@ def test_every_finite_amax_lands_on_448_in_the_hardware_converter():
     qo, so = oracle.cast_colwise_transposed(xt)
     assert torch.equal(qt.cpu().view(torch.uint8), qo) and bits_equal(st.cpu().reshape(-1), so)
     assert torch.equal(qt.cpu().view(torch.uint8), q.cpu().view(torch.uint8))  # same bytes either way
+
+
+def test_pytorchs_gpu_division_by_a_scalar_is_the_product_with_the_inverse():
+    """What `torch.clamp(amax_t.float(), min=EPS) / FP8_MAX` (lingua/float8.py:44) gives on this GPU, for every
+    non-negative bf16 amax: PyTorch's GPU kernel multiplies by fp32(1/448), its CPU kernel divides, and the two differ
+    in the last bit for a good third of the amaxes.  This pins the oracle's "times_inverse" rule against PyTorch's own
+    kernel; the default rule is pinned against the CPU kernel in tests/test_oracle_cast.py."""
+    bits = torch.arange(0, 0x7F81, dtype=torch.int32).to(torch.int16).view(torch.bfloat16)
+    on_gpu = (torch.clamp(bits.cuda().float(), min=1e-12) / 448.0).cpu()
+    on_cpu = torch.clamp(bits.float(), min=1e-12) / 448.0
+    assert bits_equal(oracle.scale_from_amax(bits), on_cpu)
+    with oracle.scale_rule("times_inverse"):
+        assert bits_equal(oracle.scale_from_amax(bits), on_gpu)
+    differ = (on_gpu.view(torch.int32) != on_cpu.view(torch.int32)).float().mean().item()
+    assert 0.2 < differ < 0.6
+
+
+@pytest.mark.parametrize("shape", [(4096, 2048), (777, 1000), (64, 11008), (3, 8)])
+def test_casts_under_the_gpu_division_rule_equal_pytorchs_own_gpu_ops(shape, gpu_division_rule):
+    """With `lingua_amd.set_scale_rule("times_inverse")` every layout's bytes and scales equal, bit for bit, what the
+    reference's op chain (oracle.recipe_torch issues it op for op) gives when PyTorch runs it on this GPU -- and the
+    oracle under the same rule."""
+    from oracle import recipe_torch as rt
+    from lingua_amd import ops
+    x = seeded_bf16(shape, 1.0, seed=shape[0] + shape[1])
+    x[0, 0] = 0
+    if shape[0] > 2:
+        x[1] = 0                      # a zero row: the floor of the clamp under this rule
+    xd = x.cuda()
+    # row-wise
+    q, s, a = ops.cast_rowwise(xd)
+    q_t, s_t = rt.scale(xd, rt.row_amax(xd))
+    assert bits_equal(q.view(torch.uint8), q_t.view(torch.uint8)) and bits_equal(s.reshape(-1), s_t.reshape(-1))
+    q_o, s_o, _ = oracle.cast_rowwise(x)
+    assert torch.equal(q.cpu().view(torch.uint8), q_o) and bits_equal(s.cpu().reshape(-1), s_o)
+    # an amax of the caller's, fp32
+    amax32 = rt.row_amax(xd).float() * 1.5
+    q, s = ops.cast_rowwise_given_amax(xd, amax32)
+    q_t, s_t = rt.scale(xd, amax32)
+    assert bits_equal(q.view(torch.uint8), q_t.view(torch.uint8)) and bits_equal(s.reshape(-1), s_t.reshape(-1))
+    # column-wise, transposed (the wgrad operands)
+    col = torch.zeros(shape[1], dtype=torch.float32, device="cuda")
+    ops.cast_rowwise(xd, col_amax=col)
+    q, s = ops.cast_colwise_transposed(xd, col)
+    xt = xd.t().contiguous()
+    q_t, s_t = rt.scale(xt, rt.row_amax(xt))
+    assert bits_equal(q[:, :shape[0]].contiguous().view(torch.uint8), q_t.view(torch.uint8)) and bits_equal(s.reshape(-1), s_t.reshape(-1))
+    # one scale for the tensor, both layouts
+    amax = xd.abs().amax().reshape(1, 1)
+    for transpose in (False, True):
+        q, s = ops.cast_tensorwise(xd, amax, transpose=transpose)
+        q_t, s_t = rt.scale(xt if transpose else xd, amax)
+        cols = shape[0] if transpose else shape[1]
+        assert bits_equal(q[:, :cols].contiguous().view(torch.uint8), q_t.view(torch.uint8)) and bits_equal(s.reshape(-1), s_t.reshape(-1))

@@ -700,3 +700,58 @@ def test_two_streams_keep_their_own_shared_casts():
             assert torch.equal(y1, a1(x)) and torch.equal(y3, a3(x))
         finally:
             float8.config.share_input_casts = True
+
+
+@pytest.mark.parametrize("shape", [(4096, 2048, 2048, False), (2000, 1024, 4096, True)])
+def test_forward_and_dgrad_against_the_reference_op_chain_run_on_this_gpu(shape, gpu_division_rule):
+    """The reference's sequence of ATen ops, issued op for op by oracle.recipe_torch (abs / amax / clamp / div /
+    reciprocal / mul / to(float8_e4m3fn), lingua/float8.py:43-47,86-87,115-118), run by PyTorch's own kernels on this
+    GPU, with the product through torch._scaled_mm exactly as lingua/float8.py:65-73 calls it.  Under the division
+    rule of PyTorch's GPU kernel (`set_scale_rule("times_inverse")`; under the default rule, the CPU kernel's, half
+    the scales differ in their last bit and 0.03-0.1 % of the bytes with them) the fp8 bytes and scales of this library
+    must equal that chain's bit for bit; y and dX must agree an order of magnitude inside the benchmark's tolerance
+    (the two products run on the same matrix instructions)."""
+    from golden_util import bits_equal
+    from lingua_amd import ops
+    import lingua_amd.float8 as f8
+    M, K, N, with_bias = shape
+    x = seeded_bf16((M, K), 1.0, seed=11).cuda()
+    w = seeded_bf16((N, K), 0.02, seed=12).cuda()
+    b = seeded_bf16((N,), 0.5, seed=13).cuda() if with_bias else None
+    gy = seeded_bf16((M, N), 1e-2, seed=14).cuda()
+
+    def mm(q1, s1, q2_t, s2_t, bias=None):
+        return torch._scaled_mm(q1, q2_t.t(), scale_a=s1, scale_b=s2_t.t(), bias=bias, out_dtype=torch.bfloat16,
+                                use_fast_accum=True)
+
+    # forward: both operands row-wise
+    qx_ref, sx_ref = rt.scale(x, rt.row_amax(x))
+    qw_ref, sw_ref = rt.scale(w, rt.row_amax(w))
+    qx, sx, ax = ops.cast_rowwise(x)
+    qw, sw, aw = ops.cast_rowwise(w)
+    assert bits_equal(qx.view(torch.uint8), qx_ref.view(torch.uint8)) and bits_equal(sx.reshape(-1), sx_ref.reshape(-1))
+    assert bits_equal(qw.view(torch.uint8), qw_ref.view(torch.uint8)) and bits_equal(sw.reshape(-1), sw_ref.reshape(-1))
+    assert bits_equal(ax.reshape(-1), rt.row_amax(x).reshape(-1))
+    try:
+        y_ref = mm(qx_ref, sx_ref, qw_ref, sw_ref, b)
+    except (RuntimeError, NotImplementedError) as e:
+        pytest.skip(f"torch._scaled_mm with row-wise scales is not available here: {e}")
+    lin = f8.Fp8Linear(K, N, bias=with_bias, dtype=torch.bfloat16, device="cuda")
+    with torch.no_grad():
+        lin.weight.copy_(w)
+        if with_bias:
+            lin.bias.copy_(b)
+    xg = x.clone().requires_grad_(True)
+    y = lin(xg)
+    assert rel_l2(y, y_ref) <= 1e-4
+    # dgrad: grad_out row-wise, the weight with one scale for the whole tensor, transposed copy
+    y.backward(gy)
+    wt = w.t().contiguous()
+    amax_wt = rt.tensor_amax_from_rows(rt.row_amax(w), K)
+    qg_ref, sg_ref = rt.scale(gy, rt.row_amax(gy))
+    qwt_ref, swt_ref = rt.scale(wt, amax_wt)
+    qwt, swt = ops.cast_tensorwise(w, ops.amax_reduce(aw), transpose=True)
+    assert bits_equal(qwt.view(torch.uint8), qwt_ref.view(torch.uint8))
+    assert bits_equal(swt.reshape(-1), swt_ref[:1].reshape(-1))
+    dx_ref = mm(qg_ref, sg_ref, qwt_ref, swt_ref)
+    assert rel_l2(xg.grad, dx_ref) <= 1e-4

@@ -239,3 +239,8 @@ def test_fused_feed_forward_takes_the_norm_output_already_quantised():
     assert n_apart == 4 and n_shared == 3          # x + three weights against the three weights only
     for a, b in zip(got, want):
         assert torch.equal(a.view(torch.int16), b.view(torch.int16))
+
+
+def test_norm_cast_under_the_gpu_division_rule(gpu_division_rule):
+    for shape in [(5, 264), (300, 1000), (17, 4096), (9, 8192)]:
+        test_norm_and_cast(shape, torch.bfloat16, True)

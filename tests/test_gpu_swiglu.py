@@ -254,3 +254,11 @@ def test_7b_gate_shapes_properties():
     for got, want in ((g1, a1.grad), (g3, a3.grad)):
         d = bf16_ulp_distance(got.cpu(), want.cpu())
         assert int(d.max()) <= MAX_ULPS and float((d == 0).float().mean()) >= ULP_EXACT_FRACTION
+
+
+def test_gate_casts_under_the_gpu_division_rule(gpu_division_rule):
+    """The fused gate kernels take their scales from the same helper as the plain casts: under the other division rule
+    their bytes and scales follow the oracle under that rule."""
+    for shape in [(5, 264), (33, 4096), (21, 11008), (3, 32768)]:
+        test_forward_gate_and_cast(shape, True)
+        test_backward_gate_and_casts(shape, True)

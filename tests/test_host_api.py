@@ -260,3 +260,23 @@ def test_converter_drops_compiled_code_like_the_reference():
     compiled(x)
     assert len(traces) == 2                    # traced afresh after the conversion
     torch._dynamo.reset()
+
+
+def test_scale_rule_switch_is_host_state_with_a_checked_argument():
+    """l8_set_scale_rule / l8_get_scale_rule: host-only state, default = the correctly rounded quotient, unknown rules
+    rejected with a message; the Python switch drops the quantised copies it holds."""
+    import lingua_amd
+    from lingua_amd import _lib, ops
+    lib = _lib.load()
+    assert lib.l8_get_scale_rule() == 0 and ops.get_scale_rule() == "divide"
+    assert lib.l8_set_scale_rule(7) != 0 and b"unknown rule" in lib.l8_last_error()
+    assert lib.l8_get_scale_rule() == 0
+    try:
+        lingua_amd.set_scale_rule("times_inverse")
+        assert lib.l8_get_scale_rule() == 1 and lingua_amd.get_scale_rule() == "times_inverse"
+        with pytest.raises(RuntimeError, match="unknown scale rule"):
+            lingua_amd.set_scale_rule("fast")
+        assert lingua_amd.get_scale_rule() == "times_inverse"
+    finally:
+        lingua_amd.set_scale_rule("divide")
+    assert lib.l8_get_scale_rule() == 0

@@ -137,3 +137,34 @@ def test_row_and_col_amax_bruteforce_and_nan():
     assert tot.isnan()
     y = x.clone(); y[5, 7] = 0
     assert oracle.amax_of_amaxes(oracle.row_amax(y)).isinf()
+
+
+def test_scale_under_the_gpu_division_rule_exhaustive_vs_numpy():
+    """ATen's GPU kernel divides a tensor by a Python scalar by multiplying with fp32(1/scalar); under
+    oracle.scale_rule("times_inverse") the oracle does the same.  Every non-negative bf16 amax against numpy float32
+    arithmetic; the rule must change the last bit of a good part of the scales (else it would pin nothing) and must
+    leave amax * (1/scale) on the code of 448 all the same.  (That PyTorch's GPU kernel really computes this product
+    is checked on the GPU, tests/test_gpu_cast.py.)"""
+    bits = np.arange(0, 0x7F81, dtype=np.uint32)
+    amax_f32 = (bits << 16).view(np.float32)
+    inv = np.float32(1.0) / np.float32(448.0)
+    with np.errstate(over="ignore"):
+        want = np.maximum(amax_f32, np.float32(1e-12)) * inv
+        quotient = np.maximum(amax_f32, np.float32(1e-12)) / np.float32(448.0)
+    amax = torch.from_numpy(amax_f32.copy()).to(torch.bfloat16)
+    with oracle.scale_rule("times_inverse"):
+        got = oracle.scale_from_amax(amax).numpy()
+        from oracle import recipe_torch as rt
+        _, chain = rt.scale(torch.zeros(amax.numel(), 1, dtype=torch.bfloat16), amax.reshape(-1, 1))
+    assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
+    assert np.array_equal(chain.numpy().reshape(-1).view(np.uint32), want.view(np.uint32))
+    differ = (got.view(np.uint32) != quotient.view(np.uint32)).mean()
+    assert 0.2 < differ < 0.6
+    assert np.abs(got.view(np.int32).astype(np.int64) - quotient.view(np.int32).astype(np.int64)).max() == 1
+    # back under the default rule the quotient is what comes out
+    assert np.array_equal(oracle.scale_from_amax(amax).numpy().view(np.uint32), quotient.view(np.uint32))
+    fin = torch.from_numpy(amax_f32[(amax_f32 >= 1e-12) & np.isfinite(amax_f32)].copy())
+    with oracle.scale_rule("times_inverse"):
+        s = oracle.scale_from_amax(fin.to(torch.bfloat16))
+    p = fin * (1.0 / s)
+    assert (oracle.e4m3fn_from_f32(p) == 0x7E).all() and float(p.max()) < 464.0 and float(p.min()) > 432.0

@@ -260,3 +260,27 @@ def test_subrow_product_oracle_reduces_to_known_cases():
     sa0[:, 2] = 0.0
     lost = qa[:, 2 * cs:3 * cs].float() @ qb[:, 2 * cs:3 * cs].float().t()
     assert torch.equal(rt.dequant_matmul(qa, sa0, qb, ones_b).float(), want - lost)
+
+
+@pytest.mark.parametrize("shape", [(5, 16), (33, 520), (64, 1000)])
+def test_c_oracle_equals_torch_chain_under_the_gpu_division_rule(shape):
+    """Both restatements under oracle.scale_rule("times_inverse"): same bytes and scales as each other in every
+    layout, and not the same as under the default rule (bf16 inputs meet e4m3's rounding ties exactly, so the last bit
+    of a scale decides bytes)."""
+    x = seeded_bf16(shape, seed=11)
+    x[0, 0] = 0
+    q0, s0, _ = oracle.cast_rowwise(x)
+    with oracle.scale_rule("times_inverse"):
+        q, s, a = oracle.cast_rowwise(x)
+        qt, st = rt.scale(x, rt.row_amax(x))
+        assert torch.equal(q, qt.view(torch.uint8)) and bits_equal(s, st.reshape(-1))
+        q2, s2 = oracle.cast_colwise_transposed(x)
+        xt = x.t().contiguous()
+        q2t, s2t = rt.scale(xt, rt.row_amax(xt))
+        assert torch.equal(q2, q2t.view(torch.uint8)) and bits_equal(s2, s2t.reshape(-1))
+        qa, sa = oracle.cast_tensorwise(x)
+        qc, sc = rt.scale(x, x.abs().amax().reshape(1, 1))
+        assert torch.equal(qa, qc.view(torch.uint8)) and bits_equal(sa, sc.reshape(-1))
+    assert not bits_equal(s, s0)
+    q1, s1, _ = oracle.cast_rowwise(x)          # the rule is back to the default outside the block
+    assert torch.equal(q1, q0) and bits_equal(s1, s0)
