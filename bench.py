@@ -703,7 +703,7 @@ def main():
         "data": "synthetic",
         "config": {"workload": "llama-7B SwiGLU MLP fwd+bwd, row-wise fp8 (configs[2])", "dim": DIM, "ffn": FFN,
                    "tokens": TOKENS, "flop_per_step": STEP_FLOP, "gemm_algo": args.algo,
-                   "wgrad": "fp8"},
+                   "wgrad": "fp8", "scale_rule": ops.get_scale_rule()},
         "frac_of_fp8_peak": round(tflops / PEAK_FP8_TFLOPS, 4),
         "roofline": roofline,
         "kernels": kernels,
