@@ -273,7 +273,7 @@ def test_against_the_scaled_mm_call_the_reference_makes(mnk):
     """`torch._scaled_mm` with row-wise scales is what the reference's matmul() calls (lingua/float8.py:65-73); on this
     GPU it is the vendor library's kernel, an independent implementation on the same matrix instructions.  On the same
     quantised operands the two bf16 results must agree far inside the benchmark's tolerance.  Both deviate from the
-    correctly rounded product in about 1 % of the elements, K = 64 or K = 16384 alike: the fp8 matrix instruction sums
+    correctly rounded product in about 1 % of the elements, K = 128 or K = 16384 alike: the fp8 matrix instruction sums
     its 64 products with roughly 12 bits below the largest of them, which no kernel above it can change -- that, not
     the order of accumulation, is why rel-L2 against the fp32 oracle sits near 2e-4 on every shape."""
     from lingua_amd import ops
