@@ -595,7 +595,7 @@ __global__ __launch_bounds__(NW * 64) void gemm_nt_stream_kernel(const GemmArgs 
   const int n_tail = !sk ? 0 : (helper ? (loc < r_tail ? (r_tail - loc + n_help - 1) / n_help : 0) : 1);  // pieces of this workgroup
   const int n_seg = sk ? n_rounds : (loc < cnt ? (cnt - loc + W - 1) / W : 0);                              // whole tiles
   if (n_seg + n_tail == 0) return;
-  [[maybe_unused]] uint64_t prof[16] = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+  [[maybe_unused]] uint64_t prof[24] = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
   if (L8_GEMM_PROF) {
     prof[0] = __builtin_amdgcn_s_memrealtime();
     prof[5] = __builtin_readcyclecounter();
@@ -609,7 +609,38 @@ __global__ __launch_bounds__(NW * 64) void gemm_nt_stream_kernel(const GemmArgs 
     m0 = (first_m + in_grp % gsz) * BM;
     n0 = (in_grp / gsz) * BN;
   };
-  auto tile_of = [&](int seg, int &m0, int &n0) { tile_at(first + loc + seg * W, m0, n0); };
+  // The whole tiles of a workgroup are first + loc, + W, + 2 W, ...: two cursors walk that sequence, one for the loader
+  // (two K tiles ahead) and one for the multiply / store side, each holding (group, index in the group) so that a
+  // tile's origin costs a shift and a mask.  (tile_at's divisions, a hundred dependent instructions each between the
+  // scalar and the vector unit, took a thousand cycles per tile with idle matrix cores, on either side.)
+  static_assert((GROUP_M & (GROUP_M - 1)) == 0, "GROUP_M is a power of two");
+  struct TileCursor { int grp, in_grp; };
+  const int per_group_c = GROUP_M * p.tiles_n;
+  TileCursor cur_mul, cur_ld;
+  {
+    const int lin0 = first + loc;
+    cur_mul.grp = lin0 / per_group_c;
+    cur_mul.in_grp = lin0 - cur_mul.grp * per_group_c;
+    cur_ld = cur_mul;
+  }
+  auto cursor_origin = [&](const TileCursor &c, int &m0, int &n0) {
+    const int first_m = c.grp * GROUP_M;
+    const int left = p.tiles_m - first_m;
+    if (left >= GROUP_M) {
+      m0 = (first_m + (c.in_grp & (GROUP_M - 1))) * BM;
+      n0 = (c.in_grp / GROUP_M) * BN;
+    } else {  // the last, shorter group of tile rows
+      m0 = (first_m + c.in_grp % left) * BM;
+      n0 = (c.in_grp / left) * BN;
+    }
+  };
+  auto cursor_step = [&](TileCursor &c) {
+    c.in_grp += W;
+    while (c.in_grp >= per_group_c) {
+      c.in_grp -= per_group_c;
+      ++c.grp;
+    }
+  };
   // piece pc of the tail (highest tile first): tile origin, K-tile range [kb, ke); returns the tail tile's number
   // piece pc of this workgroup's tail: the tail tile's number (tile origin in m0, n0); every piece of a workgroup
   // covers the same K tiles [piece_kb, piece_ke)
@@ -660,7 +691,8 @@ __global__ __launch_bounds__(NW * 64) void gemm_nt_stream_kernel(const GemmArgs 
     if (seg < n_seg + n_tail) {
       int m0, n0;
       if (!SK || seg < n_seg) {
-        tile_of(seg, m0, n0);
+        cursor_origin(cur_ld, m0, n0);  // ld_open is called for seg = 0, 1, 2, ... in turn
+        cursor_step(cur_ld);
         if (SK) ld_ke = KT;
       } else {
         piece_of(seg - n_seg, m0, n0);
@@ -1074,16 +1106,36 @@ __global__ __launch_bounds__(NW * 64) void gemm_nt_stream_kernel(const GemmArgs 
       t_loop = __builtin_readcyclecounter();
     }
     int m0, n0;
-    tile_of(seg, m0, n0);
+    cursor_origin(cur_mul, m0, n0);
+    cursor_step(cur_mul);
+    if (L8_GEMM_PROF && seg > 0) prof[17] += __builtin_readcyclecounter() - t_loop;
     if (seg > 0) lane_consts();
+    if (L8_GEMM_PROF && seg > 0) {
+      asm volatile("" : "+v"(a_voff[0]), "+v"(b_voff[1]), "+v"(foff[1][1]));
+      prof[18] += __builtin_readcyclecounter() - t_loop;
+    }
     load_scales(m0, n0);
     int kt = 0;
+    if (L8_GEMM_PROF && seg > 0) prof[16] += __builtin_readcyclecounter() - t_loop;  // tile origin, lane constants, scale requests
     if (seg > 0) {
       // The first barrier after the N_STORES stores of a C tile: they are younger than the panels waited for
       // and the counter retires in order, so the count allows for them (waiting for the stores themselves would
       // stall the start of every tile).
       trip(integral_constant<int, N_STORES + PEND>{});
       kt = 1;
+      if (L8_GEMM_PROF && !SK && KT > 4) {  // the first trips after a stored tile, one by one
+        const uint64_t ta = __builtin_readcyclecounter();
+        prof[12] += ta - t_loop;
+        trip(integral_constant<int, PEND>{});
+        const uint64_t tb = __builtin_readcyclecounter();
+        prof[13] += tb - ta;
+        trip(integral_constant<int, PEND>{});
+        const uint64_t tc = __builtin_readcyclecounter();
+        prof[14] += tc - tb;
+        trip(integral_constant<int, PEND>{});
+        prof[15] += __builtin_readcyclecounter() - tc;
+        kt = 4;
+      }
     }
 #pragma unroll 1
     for (; kt < KT; ++kt) trip(integral_constant<int, PEND>{});
@@ -1147,8 +1199,8 @@ __global__ __launch_bounds__(NW * 64) void gemm_nt_stream_kernel(const GemmArgs 
     prof[6] = n_seg;
     prof[7] = ((uint64_t)__builtin_amdgcn_s_getreg(63508) << 32) | (uint32_t)__builtin_amdgcn_s_getreg(63492);  // XCC_ID, HW_ID
     if (threadIdx.x == 0 && p.dbg) {
-      uint64_t *d = p.dbg + (int64_t)blockIdx.x * 16;
-      for (int i = 0; i < 16; ++i) d[i] = prof[i];
+      uint64_t *d = p.dbg + (int64_t)blockIdx.x * 24;
+      for (int i = 0; i < 24; ++i) d[i] = prof[i];
     }
   }
 #else
