@@ -657,9 +657,11 @@ __global__ __launch_bounds__(NW * 64) void gemm_nt_stream_kernel(const GemmArgs 
   // g = wave * NL + i.  For the A panel LDS row = tile row.  For the B panel LDS row r = span*128 + tn*32 + j
   // holds tile row span*128 + 4*cg(j) + tn with cg(j) = 2*(j & 15) + (j >> 4): within a group (8 consecutive j)
   // the rows are 8 apart, and the group's first row is span*128 + 64*(g & 1) + 4*((g >> 1) & 1) + (g%16)/4.
-  // The per-lane constants of the K loop are formed afresh, from an opaque copy of the lane number, in front of
-  // every tile's K loop: values that lived across the conversion of the C tile (the point of highest register
-  // pressure) were the ones the allocator chose to spill, and it reloaded them inside the K loop.
+  // The per-lane constants of the K loop (ten registers) are formed from an opaque copy of the lane number.  In the
+  // instantiation that shares K ranges out they are formed afresh in front of every tile's K loop: there, values that
+  // lived across the conversion of the C tile (the point of highest register pressure) were the ones the allocator
+  // chose to spill, and it reloaded them inside the K loop.  The others have the registers to keep them (two hundred
+  // cycles per tile with idle matrix cores otherwise).
   uint32_t a_voff[2], b_voff[2], foff[2][2];
   int chunk_even, chunk_odd;
   auto lane_consts = [&]() {
@@ -790,6 +792,17 @@ __global__ __launch_bounds__(NW * 64) void gemm_nt_stream_kernel(const GemmArgs 
   int seg_sa[2] = {0, 0};
   v4i seg_sb = {0, 0, 0, 0};
   [[maybe_unused]] v2i seg_bias = {0, 0};
+  // The descriptors cover the whole scale (bias) vectors and live as long as the kernel: a tile's requests then cost a
+  // few address instructions (with a descriptor per tile, sixty scalar instructions at one per five cycles stood
+  // between two tiles).  Rows past M and columns past N fall outside the range and read as zero; M, N < 2^29 here
+  // (the host checks) so the byte offsets fit.
+  const __amdgpu_buffer_rsrc_t rsSa = make_rsrc(p.sa, p.sa_row ? (uint32_t)p.M * 4u : 4u);
+  const __amdgpu_buffer_rsrc_t rsSb = make_rsrc(p.sb, p.sb_row ? (uint32_t)p.N * 4u : 4u);
+  [[maybe_unused]] const __amdgpu_buffer_rsrc_t rsBias = make_rsrc(HAS_BIAS ? (const void *)p.bias : (const void *)p.sb, (uint32_t)p.N * 2u);
+  // a scale that is one number for the whole operand is read once (read per tile, between the stores of one tile
+  // and the K loop of the next, it was a vector load whose result was copied at once: a wait for every store)
+  const int sa_one = p.sa_row ? 0 : __builtin_amdgcn_readfirstlane(__float_as_int(p.sa[0]));
+  const int sb_one = p.sb_row ? 0 : __builtin_amdgcn_readfirstlane(__float_as_int(p.sb[0]));
   auto load_scales = [&](int m0, int n0) {
     // lane-derived values are formed afresh from an opaque copy of the lane number wherever a tile's prologue or
     // epilogue needs them, so that none of them lives across a K loop
@@ -797,25 +810,18 @@ __global__ __launch_bounds__(NW * 64) void gemm_nt_stream_kernel(const GemmArgs 
     asm volatile("" : "+v"(l));
     const int l31 = l & 31;
     const int cg = 2 * (l31 & 15) + (l31 >> 4);  // this lane's group of four output columns (of its wave's 32)
-    const int64_t sa_left = (int64_t)(p.M - m0) * 4, sb_left = (int64_t)(p.N - n0) * 4;
     if (p.sa_row) {
-      const __amdgpu_buffer_rsrc_t rsSa = make_rsrc(p.sa + m0, sa_left < 0x7fffffff ? (uint32_t)sa_left : 0x7fffffffu);
-      seg_sa[0] = __builtin_amdgcn_raw_buffer_load_b32(rsSa, (wm * WROWS + l) * 4, 0, 0);
-      if constexpr (TM == 4) seg_sa[1] = __builtin_amdgcn_raw_buffer_load_b32(rsSa, (wm * WROWS + 64 + l) * 4, 0, 0);
+      seg_sa[0] = __builtin_amdgcn_raw_buffer_load_b32(rsSa, (wm * WROWS + l) * 4, m0 * 4, 0);
+      if constexpr (TM == 4) seg_sa[1] = __builtin_amdgcn_raw_buffer_load_b32(rsSa, (wm * WROWS + 64 + l) * 4, m0 * 4, 0);
     } else {
-      seg_sa[0] = seg_sa[1] = __float_as_int(p.sa[0]);
+      seg_sa[0] = seg_sa[1] = sa_one;
     }
     if (p.sb_row) {
-      const __amdgpu_buffer_rsrc_t rsSb = make_rsrc(p.sb + n0, sb_left < 0x7fffffff ? (uint32_t)sb_left : 0x7fffffffu);
-      seg_sb = __builtin_amdgcn_raw_buffer_load_b128(rsSb, (wn * 128 + 4 * cg) * 4, 0, 0);
+      seg_sb = __builtin_amdgcn_raw_buffer_load_b128(rsSb, (wn * 128 + 4 * cg) * 4, n0 * 4, 0);
     } else {
-      const int bits = __float_as_int(p.sb[0]);
-      seg_sb = v4i{bits, bits, bits, bits};
+      seg_sb = v4i{sb_one, sb_one, sb_one, sb_one};
     }
-    if constexpr (HAS_BIAS) {
-      const __amdgpu_buffer_rsrc_t rsBias = make_rsrc(p.bias + n0, (uint32_t)((p.N - n0) * 2));
-      seg_bias = __builtin_amdgcn_raw_buffer_load_b64(rsBias, (wn * 128 + 4 * cg) * 2, 0, 0);
-    }
+    if constexpr (HAS_BIAS) seg_bias = __builtin_amdgcn_raw_buffer_load_b64(rsBias, (wn * 128 + 4 * cg) * 2, n0 * 2, 0);
   };
   // (A compute unit drains its stores at about 16 bytes per clock: the 128 KiB of a C tile keep it busy for some
   // 8000 cycles, of which the conversion below hides about half.)
@@ -967,6 +973,13 @@ __global__ __launch_bounds__(NW * 64) void gemm_nt_stream_kernel(const GemmArgs 
   };
 
   auto store_tile = [&](int m0, int n0, auto parts_tag) {
+    // The tile's scales (and bias) are used here, on every path, so that the compiler's bookkeeping of outstanding
+    // loads knows them landed whichever conversion follows.  Without it the path "requested as a row of scales,
+    // converted with a scalar scale" (which no launch takes) left their registers marked as awaited, and the first
+    // write to one of them between two tiles got an s_waitcnt vmcnt(0) -- a wait for every store of the tile just
+    // written, some 600 cycles with idle matrix cores.
+    if constexpr (HAS_BIAS) asm volatile("" : : "v"(seg_sa[0]), "v"(seg_sa[1]), "v"(seg_sb), "v"(seg_bias));
+    else asm volatile("" : : "v"(seg_sa[0]), "v"(seg_sa[1]), "v"(seg_sb));
     if (p.sb_row) store_tile_as(m0, n0, parts_tag, std::true_type{});
     else store_tile_as(m0, n0, parts_tag, std::false_type{});
   };
@@ -1109,7 +1122,7 @@ __global__ __launch_bounds__(NW * 64) void gemm_nt_stream_kernel(const GemmArgs 
     cursor_origin(cur_mul, m0, n0);
     cursor_step(cur_mul);
     if (L8_GEMM_PROF && seg > 0) prof[17] += __builtin_readcyclecounter() - t_loop;
-    if (seg > 0) lane_consts();
+    if (SK && seg > 0) lane_consts();
     if (L8_GEMM_PROF && seg > 0) {
       asm volatile("" : "+v"(a_voff[0]), "+v"(b_voff[1]), "+v"(foff[1][1]));
       prof[18] += __builtin_readcyclecounter() - t_loop;
@@ -1369,7 +1382,9 @@ static int gemm_nt_impl(const void *A, const void *B, int64_t M, int64_t N, int6
   if (kAlgos[algo - 1].persistent) {
     // the persistent kernel stores 16 aligned bytes (eight columns) per lane and reads the row scales 16 bytes
     // at a time; operands that do not allow that go to the plain kernel with the same tile shape
+    // (and addresses its scale vectors with 32-bit byte offsets)
     const bool ok = N % 8 == 0 && ldc % 8 == 0 && ((uintptr_t)C % 16) == 0 && ldc < (1LL << 22) &&
+                    M < (1LL << 29) && N < (1LL << 29) &&
                     (sa_mode != L8_SCALE_ROW || ((uintptr_t)sa % 16) == 0) &&
                     (sb_mode != L8_SCALE_ROW || ((uintptr_t)sb % 16) == 0) &&
                     (bias == nullptr || (((uintptr_t)bias % 8) == 0 && kAlgos[algo - 1].fn_bias != nullptr));
