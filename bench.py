@@ -373,8 +373,54 @@ def more_extras(torch, dev, args):
     torch.cuda.empty_cache()
     res["config4_outlier_stress"] = dict(fig, what="4096->11008 linear on Student-t(3) activations, 0.1 % of channels x100, "
                                          "1 % zero rows: SNR of the quantised x and rel-L2 of y against the fp32 product")
+    res["parity"] = parity_figures(torch, dev)
+    torch.cuda.empty_cache()
     res["llama1b"] = measure_llama1b(torch, dev, steps=5, warmup=2, fused_too=True)
     return res
+
+
+def parity_figures(torch, dev):
+    """Not a timing: how this library's results sit beside what PyTorch itself computes on this GPU for configs[0]
+    (x [4096,2048] ~ N(0,1), W [2048,2048] ~ N(0,0.02^2), seed 0).  (1) the product against torch._scaled_mm with
+    row-wise scales -- the call the reference makes -- on the same quantised operands; (2) the two readings of
+    `clamp(amax) / 448`: the correctly rounded quotient (ATen's CPU kernel, this library's default) against the product
+    with fp32(1/448) (ATen's GPU kernel): scales and bytes that differ, and what that does to y."""
+    import lingua_amd
+    from lingua_amd import ops
+    from bench_workloads import seeded_bf16, rel_l2
+    x = seeded_bf16((4096, 2048), 1.0, seed=0).to(dev)
+    w = seeded_bf16((2048, 2048), 0.02, seed=1).to(dev)
+    out = {}
+    qx, sx, _ = ops.cast_rowwise(x)
+    qw, sw, _ = ops.cast_rowwise(w)
+    y = ops.gemm_nt(qx, qw, sx, sw)
+    try:
+        ref = torch._scaled_mm(qx, qw.t(), scale_a=sx.reshape(-1, 1), scale_b=sw.reshape(1, -1), out_dtype=torch.bfloat16,
+                               use_fast_accum=True)
+        out["gemm_vs_torch_scaled_mm"] = {"rel_l2": float(f"{rel_l2(y, ref):.3e}"),
+                                          "elements_differing": float(f"{(y != ref).float().mean().item():.3e}")}
+    except (RuntimeError, NotImplementedError) as exc:
+        out["gemm_vs_torch_scaled_mm"] = {"error": str(exc)[:200]}
+    try:
+        lingua_amd.set_scale_rule("times_inverse")
+        qx2, sx2, _ = ops.cast_rowwise(x)
+        qw2, sw2, _ = ops.cast_rowwise(w)
+        y2 = ops.gemm_nt(qx2, qw2, sx2, sw2)
+        # PyTorch's own kernels on this GPU, op for op as lingua/float8.py:43-47 issues them
+        s_t = torch.clamp(x.abs().amax(dim=-1, keepdim=True).float(), min=1e-12) / 448.0
+        q_t = (x * s_t.reciprocal()).to(torch.float8_e4m3fn)
+    finally:
+        lingua_amd.set_scale_rule("divide")
+    out["division_rule"] = {
+        "scales_differing": round((sx.view(torch.int32) != sx2.view(torch.int32)).float().mean().item(), 4),
+        "bytes_differing": float(f"{(qx.view(torch.uint8) != qx2.view(torch.uint8)).float().mean().item():.3e}"),
+        "rel_l2_of_y_between_rules": float(f"{rel_l2(y2, y):.3e}"),
+        "times_inverse_equals_torch_gpu_ops": bool(torch.equal(q_t.view(torch.uint8), qx2.view(torch.uint8))
+                                                   and torch.equal(s_t.view(torch.int32), sx2.view(torch.int32))),
+        "divide_equals_torch_gpu_ops": bool(torch.equal(q_t.view(torch.uint8), qx.view(torch.uint8))
+                                            and torch.equal(s_t.view(torch.int32), sx.view(torch.int32))),
+    }
+    return out
 
 
 def bump_versions(torch, params):
