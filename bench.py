@@ -358,7 +358,7 @@ def extras(torch, mlp, timed, args):
 
 
 def more_extras(torch, dev, args):
-    """The other measurements the survey asks for, each freed before the next: one Fp8Linear forward+backward, the
+    """The other measurements of the benchmark, each freed before the next: one Fp8Linear forward+backward, the
     config-4 outlier-stress figures (row-wise against tensor-wise scaling) and the Llama-1B-shaped step."""
     res = {}
     res["linear7b"] = measure_linear7b(args, torch, dev)
