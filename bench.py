@@ -599,10 +599,17 @@ def main():
         qa, sa, _ = ops.cast_rowwise(a)
         qb, sb, _ = ops.cast_rowwise(b)
         out = torch.empty(M, N, dtype=torch.bfloat16, device=dev)
-        for _ in range(args.launches):
+        warm = min(10, args.launches // 2)   # launches before the timed ones (the clock settles under load)
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        for i in range(args.launches):
+            if i == warm:
+                e0.record()
             ops.gemm_nt(qa, qb, sa, sb, algo=args.algo, out=out)
+        e1.record()
         torch.cuda.synchronize()
+        avg_ms = e0.elapsed_time(e1) / (args.launches - warm)
         print(json.dumps({"kernel_only": "gemm", "M": M, "N": N, "K": K, "launches": args.launches,
+                          "avg_ms": round(avg_ms, 4), "TFLOP/s": round(2 * M * N * K / avg_ms / 1e9, 1),
                           "flop_per_launch": 2 * M * N * K,
                           "algorithmic_bytes": M * K + N * K + 2 * M * N + 4 * (M + N)}))
         return

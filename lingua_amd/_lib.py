@@ -9,7 +9,9 @@ import os
 import threading
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(_HERE, "liblingua_fp8.so")
+# LINGUA_FP8_LIB names another build of the library (a tuning variant made with `python -m lingua_amd.build` under the
+# same variable); unset, the library next to this file is the one that is loaded.
+LIB_PATH = os.environ.get("LINGUA_FP8_LIB") or os.path.join(_HERE, "liblingua_fp8.so")
 
 _i64 = ctypes.c_int64
 _int = ctypes.c_int

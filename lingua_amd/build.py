@@ -11,7 +11,9 @@ from concurrent.futures import ThreadPoolExecutor
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(_HERE, "csrc")
-LIB_PATH = os.path.join(_HERE, "liblingua_fp8.so")
+# LINGUA_FP8_LIB: where to put the library instead (a tuning variant beside the shipped one; `lingua_amd._lib` reads the
+# same variable); LINGUA_FP8_HIPCC_EXTRA: more hipcc flags for such a variant, e.g. "-DL8_STRADDLE=3 -DL8_READ_GROUPS=10".
+LIB_PATH = os.environ.get("LINGUA_FP8_LIB") or os.path.join(_HERE, "liblingua_fp8.so")
 SOURCES = ["api.cpp", "cast_kernels.hip", "gemm_kernels.hip", "swiglu_kernels.hip", "norm_kernels.hip"]
 
 OBJ_DIR = os.path.join(_HERE, "build")     # object files (ignored by git)
@@ -77,14 +79,16 @@ def _check_usage(usage) -> None:
 def build(verbose: bool = False) -> str:
     """Compiles every source (in parallel, one object each) and links the shared library."""
     hipcc = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
-    os.makedirs(OBJ_DIR, exist_ok=True)
-    objs = [os.path.join(OBJ_DIR, os.path.splitext(src)[0] + ".o") for src in SOURCES]
-    cmds = [[hipcc, *HIPCC_FLAGS, *(["-Rpass-analysis=kernel-resource-usage"] if src.endswith(".hip") else []),
+    extra = os.environ.get("LINGUA_FP8_HIPCC_EXTRA", "").split()
+    obj_dir = OBJ_DIR if not os.environ.get("LINGUA_FP8_LIB") else os.path.join(OBJ_DIR, os.path.splitext(os.path.basename(LIB_PATH))[0])
+    os.makedirs(obj_dir, exist_ok=True)
+    objs = [os.path.join(obj_dir, os.path.splitext(src)[0] + ".o") for src in SOURCES]
+    cmds = [[hipcc, *HIPCC_FLAGS, *extra, *(["-Rpass-analysis=kernel-resource-usage"] if src.endswith(".hip") else []),
              "-c", os.path.join(CSRC, src), "-o", obj] for src, obj in zip(SOURCES, objs)]
     with ThreadPoolExecutor(max_workers=min(len(cmds), os.cpu_count() or 1)) as pool:
         usages = list(pool.map(lambda c: _run(c, verbose), cmds))
     usage = {k: v for u in usages for k, v in u.items()}
-    with open(os.path.join(OBJ_DIR, "resource_usage.txt"), "w") as f:
+    with open(os.path.join(obj_dir, "resource_usage.txt"), "w") as f:
         for name in sorted(usage):
             f.write(f"{name} {usage[name]}\n")
     _check_usage(usage)
