@@ -92,9 +92,7 @@ L8_DEV __amdgpu_buffer_rsrc_t make_rsrc(const void *p, uint32_t bytes) {
 template <int AUX>
 L8_DEV void store16_aux(v4i data, __amdgpu_buffer_rsrc_t rs, uint32_t voff, int soff) {
   __builtin_amdgcn_raw_buffer_store_b128(data, rs, voff, soff, AUX);
-#ifndef L8_NO_STORE_NOP
   asm volatile("s_nop 1" : : "v"(data));  // the operand keeps every later write to these registers behind the wait
-#endif
 }
 #endif
 #define store16(data, rs, voff, soff, aux) store16_aux<aux>(data, rs, voff, soff)
