@@ -311,6 +311,13 @@ def linear_forward(a, b_t, bias, need_wgrad_stats: bool, gemm_algo: int):
     the two extra tensors are what backward needs beyond ``a`` and ``b_t``."""
     if a.dtype != torch.bfloat16 or b_t.dtype != torch.bfloat16:
         raise RuntimeError(f"Fp8LinearFn: bf16 input and weight required, got {a.dtype} and {b_t.dtype}")
+    if not a.is_cuda or a.device != b_t.device:
+        raise RuntimeError(f"Fp8LinearFn: input and weight must be on the same GPU, got {a.device} and {b_t.device} "
+                           "(there is no CPU path)")
+    if a.shape[-1] % 16 or b_t.shape[0] % 16:
+        # what torch._scaled_mm tells the reference at lingua/float8.py:65 (both of mat2's dimensions must be
+        # divisible by 16); here the forward product could run, but dgrad reduces over out_features
+        raise RuntimeError(f"Fp8LinearFn: in_features ({a.shape[-1]}) and out_features ({b_t.shape[0]}) must be multiples of 16")
     # column amaxes of `a` fall out of the row-wise pass; wgrad wants them
     _bwd_cast.clear(a)
     hit = _fwd_cast.get(a, b_t.data_ptr()) if config.share_input_casts else None

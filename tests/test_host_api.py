@@ -280,3 +280,18 @@ def test_scale_rule_switch_is_host_state_with_a_checked_argument():
     finally:
         lingua_amd.set_scale_rule("divide")
     assert lib.l8_get_scale_rule() == 0
+
+
+def test_linear_refuses_operands_it_cannot_serve_before_any_gpu_work():
+    """No CPU path, bf16 only, feature counts in multiples of 16 (the reference gets the last one from
+    torch._scaled_mm at lingua/float8.py:65): RuntimeError with the reason, raised before anything is launched."""
+    from lingua_amd.float8 import Fp8LinearFn
+    x = torch.zeros(8, 32, dtype=torch.bfloat16)
+    w = torch.zeros(48, 32, dtype=torch.bfloat16)
+    with pytest.raises(RuntimeError, match="no CPU path"):
+        Fp8LinearFn.apply(x, w, None)
+    with pytest.raises(RuntimeError, match="bf16 input and weight required"):
+        Fp8LinearFn.apply(x.float(), w, None)
+    meta_x = torch.zeros(8, 40, dtype=torch.bfloat16, device="meta")
+    with pytest.raises(RuntimeError):
+        Fp8LinearFn.apply(meta_x, torch.zeros(48, 40, dtype=torch.bfloat16, device="meta"), None)
