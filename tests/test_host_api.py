@@ -295,3 +295,15 @@ def test_linear_refuses_operands_it_cannot_serve_before_any_gpu_work():
     meta_x = torch.zeros(8, 40, dtype=torch.bfloat16, device="meta")
     with pytest.raises(RuntimeError):
         Fp8LinearFn.apply(meta_x, torch.zeros(48, 40, dtype=torch.bfloat16, device="meta"), None)
+
+
+def test_a_named_library_that_is_not_there_fails_loudly():
+    """LINGUA_FP8_LIB points lingua_amd at another build of the library (a tuning variant); a path that does not exist
+    is an error that names the path, never a silent return to the shipped library."""
+    import subprocess
+    import sys
+    code = ("import lingua_amd._lib as L\n"
+            "try:\n    L.load()\nexcept RuntimeError as e:\n    print('RuntimeError', str(e))\n")
+    env = dict(os.environ, LINGUA_FP8_LIB="/nonexistent/libl8_variant.so", PYTHONPATH=os.path.dirname(os.path.dirname(os.path.abspath(__file__))))
+    out = subprocess.run([sys.executable, "-c", code], env=env, capture_output=True, text=True, timeout=120)
+    assert "RuntimeError" in out.stdout and "/nonexistent/libl8_variant.so" in out.stdout, out.stdout + out.stderr
