@@ -455,11 +455,19 @@ constexpr int kTU = L8_TU;                   // passes (4-row units per thread)
 constexpr int kTR = kRG * 4 * kTU;           // rows of x per tile
 constexpr int kTStride = kTR + 16;           // LDS row stride in bytes
 
+#if defined(__HIP_DEVICE_COMPILE__)
+L8_DEV __amdgpu_buffer_rsrc_t make_rsrc(const void *p, uint32_t bytes) {
+  return __builtin_amdgcn_make_buffer_rsrc(const_cast<void *>(p), (short)0, (int)bytes, 0x00020000);
+}
+#endif
+constexpr int kAuxNT = 2;                      // cache policy of a buffer load: non-temporal
+
 template <bool PER_COL>
 __global__ __launch_bounds__(256) void cast_transposed_kernel(
     const uint16_t *__restrict__ x, int64_t R, int C, int64_t ldx, const void *__restrict__ amax_scalar, int amax_f32,
     const uint32_t *__restrict__ col_amax, uint8_t *__restrict__ q, int64_t ldq, float *__restrict__ scale,
     int vec_store, int scale_rule) {
+#if defined(__HIP_DEVICE_COMPILE__)  // the buffer-resource type exists in the device pass only
   __shared__ __attribute__((aligned(16))) uint8_t tile[kTC * kTStride];
   __shared__ float recips[kTC];
   const int t = threadIdx.x;
@@ -480,39 +488,59 @@ __global__ __launch_bounds__(256) void cast_transposed_kernel(
   const int rg = t / kCCH;  // which 4-row group of a pass
   const int c = c0 + cc * 8;
 
-  // issue the loads first: kTU units of 4 rows x 8 columns per thread
+  // Loads without branches, through buffer descriptors whose range check returns zeros: the amax behind the
+  // scale(s) first, the tile right behind it.  The counter of outstanding loads retires in order, so the wait for
+  // the amax leaves the tile's loads in flight, and the division and the reciprocal run under them.  (With a branch
+  // around each load the compiler waited for all of them after the fifth and again before the division.)
+  uint32_t amax_lo, amax_hi = 0;
+  if (PER_COL) {
+    const __amdgpu_buffer_rsrc_t rsAmax = make_rsrc(col_amax, (uint32_t)C * 4u);
+    amax_lo = (uint32_t)__builtin_amdgcn_raw_buffer_load_b32(rsAmax, (c0 + t % kTC) * 4, 0, 0);  // zero beyond column C
+  } else {
+    // two or four bytes (bf16 or fp32) as two halves: the upper half of a bf16 amax lies beyond the descriptor
+    const __amdgpu_buffer_rsrc_t rsAmax = make_rsrc(amax_scalar, amax_f32 ? 4u : 2u);
+    amax_lo = (uint16_t)__builtin_amdgcn_raw_buffer_load_b16(rsAmax, 0, 0, 0);
+    amax_hi = (uint16_t)__builtin_amdgcn_raw_buffer_load_b16(rsAmax, 2, 0, 0);
+  }
+  // keep the amax's load(s) here, ahead of the tile's: neither sunk to their first use nor rescheduled
+  asm volatile("" ::: "memory");
+  __builtin_amdgcn_sched_barrier(0);
+  // kTU units of 4 rows x 8 columns per thread.  The descriptor covers the tile's rows that exist, up to the last
+  // column of the last one: a row at or beyond R starts beyond it, and a chunk at or beyond column C (which would
+  // otherwise read the next row) is sent there.  The host keeps kTR * ldx * 2 below 2^31.
+  const int64_t rows_left = R - r0;
+  const uint32_t row_bytes = (uint32_t)ldx * 2u;
+  const uint32_t tile_bytes = (uint32_t)((rows_left < kTR ? (int)rows_left : kTR) - 1) * row_bytes + (uint32_t)C * 2u;
+  const __amdgpu_buffer_rsrc_t rsX = make_rsrc(x + r0 * ldx, tile_bytes);
+  const uint32_t voff = (c < C ? (uint32_t)c * 2u : tile_bytes) + (uint32_t)(rg * 4) * row_bytes;
   v4i in[kTU][4];
 #pragma unroll
   for (int u = 0; u < kTU; ++u)
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const int64_t r = r0 + (u * kRG + rg) * 4 + i;
-      if (r < R && c < C) in[u][i] = __builtin_nontemporal_load((const v4i *)(x + r * ldx + c));
-      else in[u][i] = v4i{0, 0, 0, 0};
-    }
+    for (int i = 0; i < 4; ++i)
+      in[u][i] = __builtin_amdgcn_raw_buffer_load_b128(rsX, voff, (u * kRG * 4 + i) * row_bytes, kAuxNT);
 
-  bool finite = true;
   if (PER_COL) {
+    // every wave computes the 64 scales (a branch around the division would pull the amax's load into it, behind
+    // the tile's loads); the first one keeps them
+    const float s = scale_from_amax_bits32(amax_lo, scale_rule);
+    float rc = recip_exact(s);
+    if (amax_lo >= 0x7f800000u) rc = __uint_as_float(0x7fc00000u);  // flag: slow path for this column
     if (t < kTC) {
-      const int col = c0 + t;
-      float rc = 0.0f;
-      if (col < C) {
-        const uint32_t bits = col_amax[col];
-        const float s = scale_from_amax_bits32(bits, scale_rule);
-        rc = recip_exact(s);
-        if (bits >= 0x7f800000u) rc = __uint_as_float(0x7fc00000u);  // flag: slow path for this column
-        if (rt == 0) scale[col] = s;
-      }
+      if (rt == 0 && c0 + t < C) scale[c0 + t] = s;
       recips[t] = rc;
     }
     __syncthreads();
   }
   float rcp[8];
+  bool finite = true;
   if (PER_COL) {
 #pragma unroll
     for (int j = 0; j < 8; ++j) rcp[j] = recips[cc * 8 + j];
   } else {
-    const float s = scale_from_amax_scalar(amax_scalar, amax_f32, finite, scale_rule);
+    const uint32_t amax_bits = (amax_lo | (amax_hi << 16)) & (amax_f32 ? 0x7fffffffu : 0x7fffu);  // the sign is ignored
+    finite = amax_bits < (amax_f32 ? 0x7f800000u : 0x7f80u);
+    const float s = amax_f32 ? scale_from_amax_bits32(amax_bits, scale_rule) : scale_from_amax_bits16(amax_bits, scale_rule);
     const float rc = recip_exact(s);
 #pragma unroll
     for (int j = 0; j < 8; ++j) rcp[j] = rc;
@@ -520,6 +548,7 @@ __global__ __launch_bounds__(256) void cast_transposed_kernel(
   }
 
   // convert and transpose inside the thread: column j <- rows 0..3 of each unit
+  bool all_fast = finite;
 #pragma unroll
   for (int u = 0; u < kTU; ++u)
 #pragma unroll
@@ -532,28 +561,33 @@ __global__ __launch_bounds__(256) void cast_transposed_kernel(
         const uint32_t p = (uint32_t)in[u][i][w];
         v[i] = __uint_as_float(hi ? (p & 0xffff0000u) : (p << 16)) * rcp[j];
       }
-      int packed;
-      const bool fast = PER_COL ? (rcp[j] == rcp[j]) : finite;
-      if (fast) {
-        packed = __builtin_amdgcn_cvt_pk_fp8_f32(v[0], v[1], 0, false);
-        packed = __builtin_amdgcn_cvt_pk_fp8_f32(v[2], v[3], packed, true);
-      } else {
-        // non-finite amax: redo the products with the true reciprocal (0 for inf, NaN for NaN)
-        float rc = rcp[j];
-        if (PER_COL) {
-          const uint32_t bits = col_amax[c + j < C ? c + j : 0];
-          rc = recip_exact(scale_from_amax_bits32(bits, scale_rule));
-        }
-        packed = 0;
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-          const uint32_t p = (uint32_t)in[u][i][w];
-          const float val = __uint_as_float(hi ? (p & 0xffff0000u) : (p << 16)) * rc;
-          packed |= (int)(e4m3fn_from_f32_slow(val) << (8 * i));
-        }
-      }
+      if (PER_COL && u == 0) all_fast &= rcp[j] == rcp[j];
+      int packed = __builtin_amdgcn_cvt_pk_fp8_f32(v[0], v[1], 0, false);
+      packed = __builtin_amdgcn_cvt_pk_fp8_f32(v[2], v[3], packed, true);
       *(int *)(tile + (cc * 8 + j) * kTStride + (u * kRG + rg) * 4) = packed;
     }
+  if (!all_fast) {
+    // A column whose amax is not finite: its bytes are redone from memory with the true reciprocal (0 for an
+    // infinite amax, NaN for a NaN) and the integer conversion, and replace what the line above wrote.
+#pragma unroll 1
+    for (int uj = 0; uj < kTU * 8; ++uj) {
+      const int u = uj >> 3, j = uj & 7;
+      float rc;
+      if (PER_COL) {
+        if (recips[cc * 8 + j] == recips[cc * 8 + j]) continue;
+        rc = recip_exact(scale_from_amax_bits32(col_amax[c + j < C ? c + j : 0], scale_rule));
+      } else {
+        rc = rcp[0];
+      }
+      uint32_t packed = 0;
+      for (int i = 0; i < 4; ++i) {
+        const int64_t r = r0 + (u * kRG + rg) * 4 + i;
+        const uint32_t h = (r < R && c + j < C) ? x[r * ldx + c + j] : 0u;
+        packed |= e4m3fn_from_f32_slow(bf16_bits_to_f32(h) * rc) << (8 * i);
+      }
+      *(uint32_t *)(tile + (cc * 8 + j) * kTStride + (u * kRG + rg) * 4) = packed;
+    }
+  }
   __syncthreads();
   // write out: 64 output rows (columns of x) x kTR bytes, 16 bytes per thread and step
   constexpr int SEGS = kTR / 16;  // 16-byte segments per output row
@@ -575,6 +609,7 @@ __global__ __launch_bounds__(256) void cast_transposed_kernel(
       }
     }
   }
+#endif
 }
 
 // ---------------------------------------------------------------------------
@@ -808,6 +843,7 @@ static int launch_transposed(bool per_col, const void *x, int64_t R, int64_t C, 
                              int amax_f32, const float *col_amax, void *q, int64_t ldq, float *scale, hipStream_t st) {
   const int64_t gx = ((C + kTC - 1) / kTC) * ((R + kTR - 1) / kTR), gy = 1;
   L8_REQUIRE(gx < (1LL << 31), "transposed cast: shape too large (%lld x %lld)", (long long)R, (long long)C);
+  L8_REQUIRE((int64_t)kTR * ldx * 2 < (1LL << 31), "transposed cast: row stride too large (%lld elements)", (long long)ldx);
   const int vec = (ldq % 16 == 0 && aligned(q, 16)) ? 1 : 0;
   if (per_col)
     hipLaunchKernelGGL((cast_transposed_kernel<true>), dim3((unsigned)gx, (unsigned)gy), dim3(256), 0, st,

@@ -175,6 +175,34 @@ def test_colwise_nonfinite_columns():
     assert bits_equal(s[fin], so[fin])
 
 
+@pytest.mark.parametrize("bad", [float("inf"), float("nan")])
+@pytest.mark.parametrize("amax_dtype", [torch.bfloat16, torch.float32])
+def test_transposed_casts_with_a_nonfinite_amax_over_several_tiles(bad, amax_dtype):
+    """The transposed kernels redo a column (or, tensor-wise, everything) whose amax is not finite with the
+    integer conversion: ragged shape, more than one tile in both directions, both halves of a tile's rows."""
+    from lingua_amd import ops
+    x = seeded_bf16((300, 136), seed=11)
+    x[1, 3] = bad
+    x[140, 70] = bad
+    x[299, 135] = bad
+    xd = dev(x)
+    amax = torch.tensor([[bad]], dtype=amax_dtype)
+    for tr in (False, True):
+        q, s = ops.cast_tensorwise(xd, dev(amax), transpose=tr)
+        qo, so = oracle.cast_tensorwise(x, amax, transpose=tr)
+        assert fp8_equal_mod_nan_sign(q.cpu().view(torch.uint8), qo), tr
+        s = s.cpu().reshape(-1)
+        assert torch.equal(s.isnan(), so.isnan()) and torch.equal(s.isinf(), so.isinf()), tr
+    if amax_dtype == torch.float32:
+        q, s = ops.cast_colwise_transposed(xd, ops.col_amax(xd))
+        qo, so = oracle.cast_colwise_transposed(x)
+        assert fp8_equal_mod_nan_sign(q[:, :300].cpu().view(torch.uint8), qo)
+        s = s.cpu().reshape(-1)
+        fin = so.isfinite()
+        assert not fin[3] and not fin[70] and not fin[135] and int(fin.sum()) == 133
+        assert bits_equal(s[fin], so[fin])
+
+
 from bench_workloads import outlier_stress_input  # noqa: E402
 
 
