@@ -119,7 +119,7 @@ int l8_amax_reduce(const void *amax, int64_t n, void *amax_out, void *stream);
  * (repeat_interleave of the scalar) + :43-47 (scale()) for the dgrad weight.
  *   transpose == 0 : q is [R,C] (ldq >= C);  != 0 : q is [C,R] (ldq >= R)
  *   scale    fp32 [1]
- * Requires C % 8 == 0, ldx % 8 == 0; with transpose != 0 also ldx < 2^22 elements. */
+ * Requires C % 8 == 0, ldx % 8 == 0; with transpose != 0 also ldx < 2^21 elements. */
 int l8_cast_tensorwise(const void *x, int64_t R, int64_t C, int64_t ldx,
                        const void *amax, int amax_dtype, int transpose,
                        void *q, int64_t ldq, float *scale, void *stream);
@@ -129,7 +129,7 @@ int l8_cast_tensorwise(const void *x, int64_t R, int64_t C, int64_t ldx,
  * the operand layout an fp8 wgrad needs; the reference computes wgrad in bf16 at :123).
  *   col_amax fp32 [C] column amaxes of x (from l8_cast_rowwise / l8_col_amax)
  *   q        e4m3fn [C,R], row stride ldq;  scale fp32 [C]
- * Requires C % 8 == 0, ldx % 8 == 0, ldx < 2^22 elements. */
+ * Requires C % 8 == 0, ldx % 8 == 0, ldx < 2^21 elements. */
 int l8_cast_colwise_transposed(const void *x, int64_t R, int64_t C, int64_t ldx,
                                const float *col_amax,
                                void *q, int64_t ldq, float *scale, void *stream);

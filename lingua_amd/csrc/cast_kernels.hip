@@ -507,7 +507,8 @@ __global__ __launch_bounds__(256) void cast_transposed_kernel(
   __builtin_amdgcn_sched_barrier(0);
   // kTU units of 4 rows x 8 columns per thread.  The descriptor covers the tile's rows that exist, up to the last
   // column of the last one: a row at or beyond R starts beyond it, and a chunk at or beyond column C (which would
-  // otherwise read the next row) is sent there.  The host keeps kTR * ldx * 2 below 2^31.
+  // otherwise read the next row) is sent there (the range check covers the sum of the lane's and the scalar offset, dword by
+  // dword).  The host keeps kTR * ldx * 2 below 2^30.
   const int64_t rows_left = R - r0;
   const uint32_t row_bytes = (uint32_t)ldx * 2u;
   const uint32_t tile_bytes = (uint32_t)((rows_left < kTR ? (int)rows_left : kTR) - 1) * row_bytes + (uint32_t)C * 2u;
@@ -843,7 +844,8 @@ static int launch_transposed(bool per_col, const void *x, int64_t R, int64_t C, 
                              int amax_f32, const float *col_amax, void *q, int64_t ldq, float *scale, hipStream_t st) {
   const int64_t gx = ((C + kTC - 1) / kTC) * ((R + kTR - 1) / kTR), gy = 1;
   L8_REQUIRE(gx < (1LL << 31), "transposed cast: shape too large (%lld x %lld)", (long long)R, (long long)C);
-  L8_REQUIRE((int64_t)kTR * ldx * 2 < (1LL << 31), "transposed cast: row stride too large (%lld elements)", (long long)ldx);
+  // a tile's 256 rows within 1 GiB: then no sum of a lane's offset (up to twice the tile) and a row's scalar offset wraps
+  L8_REQUIRE((int64_t)kTR * ldx * 2 < (1LL << 30), "transposed cast: row stride too large (%lld elements)", (long long)ldx);
   const int vec = (ldq % 16 == 0 && aligned(q, 16)) ? 1 : 0;
   if (per_col)
     hipLaunchKernelGGL((cast_transposed_kernel<true>), dim3((unsigned)gx, (unsigned)gy), dim3(256), 0, st,

@@ -42,10 +42,10 @@ def test_argument_validation_happens_before_launch():
     assert lib.l8_cast_rowwise(fake, -1, 8, 8, fake, 8, fake, None, None, None, 0, None) == -1
     assert lib.l8_cast_tensorwise(fake, 4, 8, 8, None, 0, 0, fake, 8, fake, None) == -1
     assert lib.l8_cast_colwise_transposed(fake, 4, 8, 8, None, fake, 4, fake, None) == -1
-    # a tile of the transposed casts (256 rows) must fit the 2 GiB a buffer descriptor reaches
-    assert lib.l8_cast_tensorwise(fake, 4, 8, 1 << 22, fake, 0, 1, fake, 16, fake, None) == -1
+    # a tile of the transposed casts (256 rows) must stay within 1 GiB
+    assert lib.l8_cast_tensorwise(fake, 4, 8, 1 << 21, fake, 0, 1, fake, 16, fake, None) == -1
     assert "row stride too large" in _lib.last_error()
-    assert lib.l8_cast_colwise_transposed(fake, 4, 8, 1 << 22, fake, fake, 16, fake, None) == -1
+    assert lib.l8_cast_colwise_transposed(fake, 4, 8, 1 << 21, fake, fake, 16, fake, None) == -1
     assert "row stride too large" in _lib.last_error()
     # empty problems are accepted and do nothing
     assert lib.l8_cast_rowwise(None, 0, 8, 8, None, 8, None, None, None, None, 0, None) == 0
