@@ -455,13 +455,6 @@ constexpr int kTU = L8_TU;                   // passes (4-row units per thread)
 constexpr int kTR = kRG * 4 * kTU;           // rows of x per tile
 constexpr int kTStride = kTR + 16;           // LDS row stride in bytes
 
-#if defined(__HIP_DEVICE_COMPILE__)
-L8_DEV __amdgpu_buffer_rsrc_t make_rsrc(const void *p, uint32_t bytes) {
-  return __builtin_amdgcn_make_buffer_rsrc(const_cast<void *>(p), (short)0, (int)bytes, 0x00020000);
-}
-#endif
-constexpr int kAuxNT = 2;                      // cache policy of a buffer load: non-temporal
-
 template <bool PER_COL>
 __global__ __launch_bounds__(256) void cast_transposed_kernel(
     const uint16_t *__restrict__ x, int64_t R, int C, int64_t ldx, const void *__restrict__ amax_scalar, int amax_f32,
@@ -519,7 +512,7 @@ __global__ __launch_bounds__(256) void cast_transposed_kernel(
   for (int u = 0; u < kTU; ++u)
 #pragma unroll
     for (int i = 0; i < 4; ++i)
-      in[u][i] = __builtin_amdgcn_raw_buffer_load_b128(rsX, voff, (u * kRG * 4 + i) * row_bytes, kAuxNT);
+      in[u][i] = load16_nt(rsX, voff, (u * kRG * 4 + i) * row_bytes);
 
   if (PER_COL) {
     // every wave computes the 64 scales (a branch around the division would pull the amax's load into it, behind

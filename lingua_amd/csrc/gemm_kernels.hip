@@ -76,11 +76,6 @@ typedef __attribute__((address_space(3))) void *lds_ptr_t;
 
 // The buffer-resource type and the matrix-core builtins exist only in the
 // device pass; the host pass sees empty kernel bodies (it needs the symbols only).
-#if defined(__HIP_DEVICE_COMPILE__)
-L8_DEV __amdgpu_buffer_rsrc_t make_rsrc(const void *p, uint32_t bytes) {
-  return __builtin_amdgcn_make_buffer_rsrc(const_cast<void *>(p), (short)0, (int)bytes, 0x00020000);
-}
-#endif
 
 // 16-byte-per-lane buffer store with a scalar-register offset, followed by two wait states.  A vector-ALU write to
 // one of the store's data registers right behind it can reach the register before the store has read it: with two

@@ -169,6 +169,27 @@ L8_DEV RowScale row_scale(uint32_t amax_bits, int scale_rule) {
   return r;
 }
 
+// Buffer descriptor over `bytes` bytes at p (raw: no stride, no swizzle).  A load through it whose byte offset --
+// the lane's plus the scalar one -- reaches `bytes` returns zeros (dword by dword), a store there is dropped: kernels
+// use that instead of a branch around the access, which keeps the compiler's count of outstanding loads exact.
+// The type exists only in the device pass.
+#if defined(__HIP_DEVICE_COMPILE__)
+L8_DEV __amdgpu_buffer_rsrc_t make_rsrc(const void *p, uint32_t bytes) {
+  return __builtin_amdgcn_make_buffer_rsrc(const_cast<void *>(p), (short)0, (int)bytes, 0x00020000);
+}
+// one 16-byte non-temporal load: lane offset voff, scalar offset soff (bytes)
+L8_DEV v4i load16_nt(__amdgpu_buffer_rsrc_t rs, uint32_t voff, uint32_t soff) {
+  return __builtin_amdgcn_raw_buffer_load_b128(rs, (int)voff, (int)soff, 2 /* cache policy: non-temporal */);
+}
+// non-temporal stores of 16 and 8 bytes at lane offset voff (dropped beyond the descriptor's range)
+L8_DEV void store16_nt(__amdgpu_buffer_rsrc_t rs, uint32_t voff, v4i data) {
+  __builtin_amdgcn_raw_buffer_store_b128(data, rs, (int)voff, 0, 2);
+}
+L8_DEV void store8_nt(__amdgpu_buffer_rsrc_t rs, uint32_t voff, v2i data) {
+  __builtin_amdgcn_raw_buffer_store_b64(data, rs, (int)voff, 0, 2);
+}
+#endif
+
 // Workgroup-per-row kernels that produce their row on the fly (fused gate, fused
 // norm) keep column maxima in registers (packed pairs, NCHW * 4 dwords per
 // tensor) while that fits the 256-register budget of two workgroups per CU,

@@ -130,6 +130,36 @@ def test_strided_inputs_and_nonfinite_rows():
     assert torch.equal(a0.view(torch.int16), am.view(torch.int16))
 
 
+@pytest.mark.parametrize("C", [520, 3000, 6000, 11008, 14336])
+def test_nonfinite_rows_at_every_kernel_width(C):
+    """A row whose amax is infinite or NaN takes the integer conversion in a fix-up loop of its own; one width per
+    kernel variant (256 and 512 threads, one to four chunks per thread, and the two-pass kernel), forward with and
+    without the bf16 result written out, and backward.  The bytes must equal the plain row-wise cast of the kernel's own
+    bf16 output, which the C oracle pins."""
+    from lingua_amd import ops
+    R = 9
+    h1 = seeded_bf16((R, C), std=2.0, seed=C + 1)
+    h3 = seeded_bf16((R, C), std=1.5, seed=C + 2)
+    dh = seeded_bf16((R, C), std=0.01, seed=C + 3)
+    h3[1, 5] = float("inf")
+    h3[3, C - 3] = float("nan")
+    h1[5, C // 2] = float("nan")
+    dh[7, C - 9] = float("inf")
+    h1d, h3d, dhd = h1.cuda(), h3.cuda(), dh.cuda()
+    h, q, s, am = ops.swiglu_cast_rowwise(h1d, h3d, want_h=True)
+    q0, s0, a0 = ops.cast_rowwise(h)
+    assert not torch.isfinite(s.cpu().reshape(-1)[[1, 3, 5]]).any() and torch.isfinite(s.cpu().reshape(-1)[[0, 2, 4, 6, 7, 8]]).all()
+    assert torch.equal(q0.view(torch.uint8), q.view(torch.uint8)) and torch.equal(s0.view(torch.int32), s.view(torch.int32))
+    assert torch.equal(a0.view(torch.int16), am.view(torch.int16))
+    _, q2, s2, _ = ops.swiglu_cast_rowwise(h1d, h3d, want_h=False)
+    assert torch.equal(q2.view(torch.uint8), q.view(torch.uint8)) and torch.equal(s2.view(torch.int32), s.view(torch.int32))
+    g1, g3, q1, q3, s1, s3 = ops.swiglu_bwd_cast_rowwise(dhd, h1d, h3d, None, None)
+    for g, qg, sg in ((g1, q1, s1), (g3, q3, s3)):
+        q0, s0, _ = ops.cast_rowwise(g)
+        assert torch.equal(q0.view(torch.uint8), qg.view(torch.uint8)) and torch.equal(s0.view(torch.int32), sg.view(torch.int32))
+    assert not torch.isfinite(s1.cpu().reshape(-1)[[1, 3, 5, 7]]).any()
+
+
 def test_argument_errors():
     from lingua_amd import ops
     h = seeded_bf16((4, 64)).cuda()
