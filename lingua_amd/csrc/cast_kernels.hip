@@ -23,26 +23,30 @@ namespace l8 {
 constexpr int kRowBlock = 256;
 constexpr int kRowWaves = kRowBlock / 64;
 
+// Row r of x into NCH register quadruples per lane, through a descriptor over the row: a chunk at or beyond column C
+// returns zeros, and so does every chunk of a row at or beyond R (a descriptor of no bytes), so there is no branch
+// around a load and the compiler's count of outstanding loads stays exact -- which is what lets a wave wait for the
+// current row while the next one is still in flight.
+#if defined(__HIP_DEVICE_COMPILE__)
 template <int NCH>
-L8_DEV void load_row(v4i (&buf)[NCH], const uint16_t *row, int C, int lane) {
+L8_DEV void load_row(v4i (&buf)[NCH], const uint16_t *x, int64_t r, int64_t R, int64_t ldx, int C, int lane) {
+  const __amdgpu_buffer_rsrc_t rs = make_rsrc(x + (r < R ? r : 0) * ldx, r < R ? (uint32_t)C * 2u : 0u);
 #pragma unroll
-  for (int j = 0; j < NCH; ++j) {
-    const int c = j * 512 + lane * 8;
-    if (c < C) buf[j] = __builtin_nontemporal_load((const v4i *)(row + c));
-    else buf[j] = v4i{0, 0, 0, 0};
-  }
+  for (int j = 0; j < NCH; ++j) buf[j] = load16_nt(rs, (uint32_t)(j * 512 + lane * 8) * 2u, 0);
 }
+#endif
 
 template <int NCH, bool COLMAX>
 __global__ __launch_bounds__(kRowBlock, 2) void cast_rowwise_kernel(
     const uint16_t *__restrict__ x, int64_t R, int C, int64_t ldx, uint8_t *__restrict__ q, int64_t ldq,
     float *__restrict__ scale, uint16_t *__restrict__ amax_out, uint16_t *__restrict__ col_partials, int scale_rule) {
+#if defined(__HIP_DEVICE_COMPILE__)  // buffer descriptors exist in the device pass only
   extern __shared__ uint32_t lds_colmax[];  // [C/2] packed bf16 pairs when COLMAX
   // the next row is prefetched into a second register set unless that would
   // push the wave beyond 256 VGPRs (two waves per SIMD are worth more)
   constexpr bool PREFETCH = COLMAX ? (NCH <= 8) : (NCH <= 24);
   const int lane = threadIdx.x & 63;
-  const int wave = threadIdx.x >> 6;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);  // in a scalar register: the row descriptors hang on it
   const int64_t wave_stride = (int64_t)gridDim.x * kRowWaves;
   int64_t r = (int64_t)blockIdx.x * kRowWaves + wave;
 
@@ -53,11 +57,11 @@ __global__ __launch_bounds__(kRowBlock, 2) void cast_rowwise_kernel(
   }
 
   v4i cur[NCH];
-  if (r < R) load_row<NCH>(cur, x + r * ldx, C, lane);
+  load_row<NCH>(cur, x, r, R, ldx, C, lane);
   while (r < R) {
     const int64_t rn = r + wave_stride;
     v4i nxt[PREFETCH ? NCH : 1];
-    if (PREFETCH && rn < R) load_row<PREFETCH ? NCH : 1>(nxt, x + rn * ldx, C, lane);
+    if (PREFETCH) load_row<PREFETCH ? NCH : 1>(nxt, x, rn, R, ldx, C, lane);
 
     // row amax on packed pairs
     uint32_t m = 0;
@@ -84,28 +88,22 @@ __global__ __launch_bounds__(kRowBlock, 2) void cast_rowwise_kernel(
       if (scale) scale[r] = s;
       if (amax_out) amax_out[r] = (uint16_t)amax_bits;
     }
-    if (q) {
-      uint8_t *qrow = q + r * ldq;
-      if (finite) {
+    uint8_t *qrow = q ? q + r * ldq : nullptr;
+    const __amdgpu_buffer_rsrc_t rsQ = make_rsrc(qrow, q ? (uint32_t)C : 0u);  // stores beyond column C, or without q, are dropped
 #pragma unroll
-        for (int j = 0; j < NCH; ++j) {
-          const int c = j * 512 + lane * 8;
-          if (c < C) __builtin_nontemporal_store(cvt8(cur[j], recip), (v2i *)(qrow + c));
-        }
-      } else {
-#pragma unroll
-        for (int j = 0; j < NCH; ++j) {
-          const int c = j * 512 + lane * 8;
-          if (c < C) *(v2i *)(qrow + c) = cvt8_slow(cur[j], recip);
-        }
-      }
+    for (int j = 0; j < NCH; ++j) store8_nt(rsQ, (uint32_t)(j * 512 + lane * 8), cvt8(cur[j], recip));
+    if (q && !finite) {
+      // a row with a non-finite amax: redone from memory with the integer conversion, replacing the bytes above (one
+      // small loop beside the common path instead of NCH unrolled copies of that conversion inside it)
+#pragma unroll 1
+      for (int c = lane * 8; c < C; c += 512) *(v2i *)(qrow + c) = cvt8_slow(*(const v4i *)(x + r * ldx + c), recip);
     }
     if (PREFETCH) {
 #pragma unroll
       for (int j = 0; j < NCH; ++j) cur[j] = nxt[PREFETCH ? j : 0];
-    } else if (rn < R) {
+    } else {
       __builtin_amdgcn_sched_barrier(0);  // the row registers are reused: do not start the loads early
-      load_row<NCH>(cur, x + rn * ldx, C, lane);
+      load_row<NCH>(cur, x, rn, R, ldx, C, lane);
     }
     r = rn;
   }
@@ -136,6 +134,7 @@ __global__ __launch_bounds__(kRowBlock, 2) void cast_rowwise_kernel(
       __syncthreads();
     }
   }
+#endif
 }
 
 // Long rows: the four waves of a workgroup share one row (wave w owns chunks
@@ -147,17 +146,15 @@ template <int NCHW, bool COLMAX>
 __global__ __launch_bounds__(kRowBlock, (NCHW <= 4 ? 4 : (NCHW <= 8 ? 2 : 1))) void cast_rowwise_wg_kernel(
     const uint16_t *__restrict__ x, int64_t R, int C, int64_t ldx, uint8_t *__restrict__ q, int64_t ldq,
     float *__restrict__ scale, uint16_t *__restrict__ amax_out, uint16_t *__restrict__ col_partials, int scale_rule) {
+#if defined(__HIP_DEVICE_COMPILE__)  // buffer descriptors exist in the device pass only
   __shared__ uint32_t red[2][kRowWaves];
   const int lane = threadIdx.x & 63;
   const int wave = threadIdx.x >> 6;
   auto col_of = [&](int j) { return (j * kRowWaves + wave) * 512 + lane * 8; };
-  auto load = [&](v4i (&buf)[NCHW], int64_t r) {
+  auto load = [&](v4i (&buf)[NCHW], int64_t r) {  // zeros beyond column C and for a row beyond R, as in load_row
+    const __amdgpu_buffer_rsrc_t rs = make_rsrc(x + (r < R ? r : 0) * ldx, r < R ? (uint32_t)C * 2u : 0u);
 #pragma unroll
-    for (int j = 0; j < NCHW; ++j) {
-      const int c = col_of(j);
-      if (c < C) buf[j] = __builtin_nontemporal_load((const v4i *)(x + r * ldx + c));
-      else buf[j] = v4i{0, 0, 0, 0};
-    }
+    for (int j = 0; j < NCHW; ++j) buf[j] = load16_nt(rs, (uint32_t)col_of(j) * 2u, 0);
   };
   uint32_t cmax[COLMAX ? NCHW * 4 : 1];
   if (COLMAX) {
@@ -166,10 +163,10 @@ __global__ __launch_bounds__(kRowBlock, (NCHW <= 4 ? 4 : (NCHW <= 8 ? 2 : 1))) v
   }
   int64_t r = blockIdx.x;
   v4i cur[NCHW], nxt[NCHW];
-  if (r < R) load(cur, r);
+  load(cur, r);
   for (int it = 0; r < R; ++it) {
     const int64_t rn = r + gridDim.x;
-    if (rn < R) load(nxt, rn);
+    load(nxt, rn);
     uint32_t m = 0;
 #pragma unroll
     for (int j = 0; j < NCHW; ++j)
@@ -193,16 +190,14 @@ __global__ __launch_bounds__(kRowBlock, (NCHW <= 4 ? 4 : (NCHW <= 8 ? 2 : 1))) v
       if (scale) scale[r] = s;
       if (amax_out) amax_out[r] = (uint16_t)amax_bits;
     }
-    if (q) {
-      uint8_t *qrow = q + r * ldq;
+    uint8_t *qrow = q ? q + r * ldq : nullptr;
+    const __amdgpu_buffer_rsrc_t rsQ = make_rsrc(qrow, q ? (uint32_t)C : 0u);  // stores beyond column C, or without q, are dropped
 #pragma unroll
-      for (int j = 0; j < NCHW; ++j) {
-        const int c = col_of(j);
-        if (c < C) {
-          if (finite) __builtin_nontemporal_store(cvt8(cur[j], recip), (v2i *)(qrow + c));
-          else *(v2i *)(qrow + c) = cvt8_slow(cur[j], recip);
-        }
-      }
+    for (int j = 0; j < NCHW; ++j) store8_nt(rsQ, (uint32_t)col_of(j), cvt8(cur[j], recip));
+    if (q && !finite) {  // non-finite amax: redone from memory with the integer conversion, as in cast_rowwise_kernel
+#pragma unroll 1
+      for (int c = threadIdx.x * 8; c < C; c += kRowBlock * 8)
+        *(v2i *)(qrow + c) = cvt8_slow(*(const v4i *)(x + r * ldx + c), recip);
     }
 #pragma unroll
     for (int j = 0; j < NCHW; ++j) cur[j] = nxt[j];
@@ -219,6 +214,7 @@ __global__ __launch_bounds__(kRowBlock, (NCHW <= 4 ? 4 : (NCHW <= 8 ? 2 : 1))) v
             v4i{(int)cmax[j * 4], (int)cmax[j * 4 + 1], (int)cmax[j * 4 + 2], (int)cmax[j * 4 + 3]};
     }
   }
+#endif
 }
 
 // Folds the partial column maxima [n_slots, C] (bf16, one row per workgroup of a row-wise kernel) into
@@ -453,7 +449,7 @@ constexpr int kCCH = kTC / 8;                // 8-column chunks per tile row
 constexpr int kRG = 256 / kCCH;              // 4-row groups covered by the 256 threads in one pass
 constexpr int kTU = L8_TU;                   // passes (4-row units per thread)
 constexpr int kTR = kRG * 4 * kTU;           // rows of x per tile
-constexpr int kTStride = kTR + 16;           // LDS row stride in bytes
+[[maybe_unused]] constexpr int kTStride = kTR + 16;           // LDS row stride in bytes
 
 template <bool PER_COL>
 __global__ __launch_bounds__(256) void cast_transposed_kernel(
