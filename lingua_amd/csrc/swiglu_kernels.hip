@@ -18,12 +18,15 @@
 // last bits of the fp32 sigmoid: at most two bf16 ulps apart, identical for
 // more than 99.5 % of the elements (the bound the tests state); amax, scale
 // and e4m3 bytes are then exact functions of the bf16 values produced here.
-// One workgroup of 256 or 512 threads per row (wave w of W owns the 512-column
-// chunks w, w+W, ...), the layout of the long-row kernel of cast_kernels.hip;
-// the amax -> scale -> cast stage is shared with it.
+// One 256-thread workgroup per row (wave
+// w owns the 512-column chunks w, w+4, ...), the layout of the long-row kernel
+// of cast_kernels.hip; the amax -> scale -> cast stage is shared with it.
 #include "l8_common.h"
 
 namespace l8 {
+
+constexpr int kGateBlock = 256;
+constexpr int kGateWaves = kGateBlock / 64;
 
 // 1 / (1 + exp(-x)) with the hardware exp2 and reciprocal (about 1 ulp of fp32
 // each).  The library exp and the IEEE division cost ~5x the instructions and
@@ -63,29 +66,18 @@ L8_DEV void gate_bwd2(uint32_t d, uint32_t a, uint32_t b, uint32_t &g1, uint32_t
   g3 = g3l | (g3h << 16);
 }
 
-// where the backward kernel keeps its two sets of column maxima: with 512 threads (128 registers each) always in LDS
-template <int NCHW, int BLOCK>
-constexpr bool bwd_colmax_in_lds() { return BLOCK > 256 || colmax_in_lds<NCHW, 2>(); }
-template <int NCHW, int BLOCK>
-constexpr bool fwd_colmax_in_lds() { return BLOCK > 256 || colmax_in_lds<NCHW, 1>(); }
-
-// BLOCK threads per row, NCHW chunks of 8 columns per thread (256 threads up to 4096 columns, 512 beyond: see the
-// backward kernel).  The operands of a row are requested a row ahead, all 2 * NCHW loads together, through descriptors
-// over the row (zeros at or beyond column C, no branch around a load).
-template <int NCHW, bool COLMAX, int BLOCK>
-__global__ __launch_bounds__(BLOCK, BLOCK / 128) void swiglu_cast_rowwise_kernel(  // second figure: waves per SIMD
+template <int NCHW, bool COLMAX>
+__global__ __launch_bounds__(kGateBlock, 2) void swiglu_cast_rowwise_kernel(
     const uint16_t *__restrict__ h1, const uint16_t *__restrict__ h3, int64_t R, int C, int64_t ld1, int64_t ld3,
     uint16_t *__restrict__ hout, int64_t ldh, uint8_t *__restrict__ q, int64_t ldq, float *__restrict__ scale,
     uint16_t *__restrict__ amax_out, uint16_t *__restrict__ col_partials, int scale_rule) {
-#if defined(__HIP_DEVICE_COMPILE__)  // buffer descriptors exist in the device pass only
-  constexpr int WAVES = BLOCK / 64;
-  __shared__ uint32_t red[2][WAVES];
+  __shared__ uint32_t red[2][kGateWaves];
   extern __shared__ __attribute__((aligned(16))) uint8_t dyn_lds[];
-  constexpr bool CLDS = COLMAX && fwd_colmax_in_lds<NCHW, BLOCK>();
+  constexpr bool CLDS = COLMAX && colmax_in_lds<NCHW, 1>();
   v4i *lds_cm = (v4i *)dyn_lds;  // [C / 8]
   const int lane = threadIdx.x & 63;
   const int wave = threadIdx.x >> 6;
-  auto col_of = [&](int j) { return (j * WAVES + wave) * 512 + lane * 8; };
+  auto col_of = [&](int j) { return (j * kGateWaves + wave) * 512 + lane * 8; };
   uint32_t cmax[(COLMAX && !CLDS) ? NCHW * 4 : 1];
   if (COLMAX) {
 #pragma unroll
@@ -98,22 +90,20 @@ __global__ __launch_bounds__(BLOCK, BLOCK / 128) void swiglu_cast_rowwise_kernel
       }
     }
   }
-  v4i a[NCHW], b[NCHW];
-  auto request = [&](int64_t r) {
-    const uint32_t bytes = r < R ? (uint32_t)C * 2u : 0u;  // nothing is read beyond the last row
-    if (r >= R) r = 0;
-    const __amdgpu_buffer_rsrc_t rsA = make_rsrc(h1 + r * ld1, bytes), rsB = make_rsrc(h3 + r * ld3, bytes);
-#pragma unroll
-    for (int j = 0; j < NCHW; ++j) {
-      a[j] = load16_nt(rsA, (uint32_t)col_of(j) * 2u, 0);
-      b[j] = load16_nt(rsB, (uint32_t)col_of(j) * 2u, 0);
-    }
-  };
-  request(blockIdx.x);
   int it = 0;
   for (int64_t r = blockIdx.x; r < R; r += gridDim.x, ++it) {
-    const __amdgpu_buffer_rsrc_t rsH = make_rsrc(hout ? hout + r * ldh : nullptr, hout ? (uint32_t)C * 2u : 0u);
-    v4i h[NCHW];
+    v4i a[NCHW], b[NCHW], h[NCHW];
+#pragma unroll
+    for (int j = 0; j < NCHW; ++j) {
+      const int c = col_of(j);
+      if (c < C) {
+        a[j] = __builtin_nontemporal_load((const v4i *)(h1 + r * ld1 + c));
+        b[j] = __builtin_nontemporal_load((const v4i *)(h3 + r * ld3 + c));
+      } else {
+        a[j] = v4i{0, 0, 0, 0};
+        b[j] = v4i{0, 0, 0, 0};
+      }
+    }
     uint32_t m = 0;
 #pragma unroll
     for (int j = 0; j < NCHW; ++j) {
@@ -130,36 +120,28 @@ __global__ __launch_bounds__(BLOCK, BLOCK / 128) void swiglu_cast_rowwise_kernel
         for (int k = 0; k < 4; ++k) old[k] = (int)pk_absmax_u16((uint32_t)old[k], (uint32_t)h[j][k]);
         lds_cm[c / 8] = old;
       }
-      store16_nt(rsH, (uint32_t)c * 2u, h[j]);  // dropped at or beyond column C, and altogether without hout
+      if (hout && c < C) __builtin_nontemporal_store(h[j], (v4i *)(hout + r * ldh + c));
     }
     m = wave_max_u32(max(m & 0xffffu, m >> 16));
     if (lane == 0) red[it & 1][wave] = m;
     __syncthreads();
-    request(r + gridDim.x);
     uint32_t amax_bits = 0;
 #pragma unroll
-    for (int w = 0; w < WAVES; ++w) amax_bits = max(amax_bits, red[it & 1][w]);
+    for (int w = 0; w < kGateWaves; ++w) amax_bits = max(amax_bits, red[it & 1][w]);
     const RowScale rs = row_scale(amax_bits, scale_rule);
     if (threadIdx.x == 0) {
       if (scale) scale[r] = rs.s;
       if (amax_out) amax_out[r] = (uint16_t)amax_bits;
     }
-    uint8_t *qrow = q ? q + r * ldq : nullptr;
-    const __amdgpu_buffer_rsrc_t rsQ = make_rsrc(qrow, q ? (uint32_t)C : 0u);
+    if (q) {
+      uint8_t *qrow = q + r * ldq;
 #pragma unroll
-    for (int j = 0; j < NCHW; ++j) store8_nt(rsQ, (uint32_t)col_of(j), cvt8(h[j], rs.recip));
-    if (q && !rs.finite) {
-      // A row with a non-finite amax: its bytes are redone with the integer conversion and replace the ones above --
-      // one small loop beside the common path (unrolled into it, the conversion's temporaries push loop invariants
-      // into scratch memory), which forms the gate again from the operands.
-#pragma unroll 1
-      for (int c = threadIdx.x * 8; c < C; c += BLOCK * 8) {
-        const v4i x1 = *(const v4i *)(h1 + r * ld1 + c);
-        const v4i x3 = *(const v4i *)(h3 + r * ld3 + c);
-        v4i g;
-#pragma unroll
-        for (int k = 0; k < 4; ++k) g[k] = (int)gate_fwd2((uint32_t)x1[k], (uint32_t)x3[k]);
-        *(v2i *)(qrow + c) = cvt8_slow(g, rs.recip);
+      for (int j = 0; j < NCHW; ++j) {
+        const int c = col_of(j);
+        if (c < C) {
+          if (rs.finite) __builtin_nontemporal_store(cvt8(h[j], rs.recip), (v2i *)(qrow + c));
+          else *(v2i *)(qrow + c) = cvt8_slow(h[j], rs.recip);
+        }
       }
     }
   }
@@ -172,28 +154,21 @@ __global__ __launch_bounds__(BLOCK, BLOCK / 128) void swiglu_cast_rowwise_kernel
             CLDS ? lds_cm[c / 8] : v4i{(int)cmax[j * 4], (int)cmax[j * 4 + 1], (int)cmax[j * 4 + 2], (int)cmax[j * 4 + 3]};
     }
   }
-#endif
 }
 
-// BLOCK threads per row, NCHW chunks of 8 columns per thread.  Twice 256 threads for rows beyond 4096 columns: the
-// row-ahead loads below keep 3 * NCHW registers quadruples per thread beside the results held for the cast, which at
-// NCHW = 6 does not fit the 256 registers of two workgroups of 256 per compute unit (79 spilled when tried), and at
-// NCHW = 3 fits the 128 of two workgroups of 512.
-template <int NCHW, bool COLMAX, int BLOCK>
-__global__ __launch_bounds__(BLOCK, BLOCK / 128) void swiglu_bwd_cast_rowwise_kernel(  // second figure: waves per SIMD
+template <int NCHW, bool COLMAX>
+__global__ __launch_bounds__(kGateBlock, 2) void swiglu_bwd_cast_rowwise_kernel(
     const uint16_t *__restrict__ dh, const uint16_t *__restrict__ h1, const uint16_t *__restrict__ h3, int64_t R, int C,
     int64_t lddh, int64_t ld1, int64_t ld3, uint16_t *__restrict__ g1out, uint16_t *__restrict__ g3out, int64_t ldg,
     uint8_t *__restrict__ q1, uint8_t *__restrict__ q3, int64_t ldq, float *__restrict__ scale1,
     float *__restrict__ scale3, uint16_t *__restrict__ col_partials1, uint16_t *__restrict__ col_partials3, int scale_rule) {
-#if defined(__HIP_DEVICE_COMPILE__)  // buffer descriptors exist in the device pass only
-  constexpr int WAVES = BLOCK / 64;
-  __shared__ uint32_t red[2][2][WAVES];
+  __shared__ uint32_t red[2][2][kGateWaves];
   extern __shared__ __attribute__((aligned(16))) uint8_t dyn_lds[];
-  constexpr bool CLDS = COLMAX && bwd_colmax_in_lds<NCHW, BLOCK>();
+  constexpr bool CLDS = COLMAX && colmax_in_lds<NCHW, 2>();
   v4i *lds_cm1 = (v4i *)dyn_lds, *lds_cm3 = lds_cm1 + C / 8;  // [C / 8] each
   const int lane = threadIdx.x & 63;
   const int wave = threadIdx.x >> 6;
-  auto col_of = [&](int j) { return (j * WAVES + wave) * 512 + lane * 8; };
+  auto col_of = [&](int j) { return (j * kGateWaves + wave) * 512 + lane * 8; };
   uint32_t cmax1[(COLMAX && !CLDS) ? NCHW * 4 : 1], cmax3[(COLMAX && !CLDS) ? NCHW * 4 : 1];
   if (COLMAX) {
 #pragma unroll
@@ -206,36 +181,23 @@ __global__ __launch_bounds__(BLOCK, BLOCK / 128) void swiglu_bwd_cast_rowwise_ke
       }
     }
   }
-  // All 3 * NCHW loads of a row go out together, through descriptors over that row (a chunk at or beyond column C
-  // returns zeros; no branch around a load), and a row ahead: behind the barrier of the row before, in front of its
-  // casts.  (One chunk at a time, loaded where it was consumed, left 48 bytes per thread in flight and the kernel
-  // waiting for memory latency NCHW times per row.)
-  v4i d[NCHW], a[NCHW], b[NCHW];
-  auto request = [&](int64_t r) {
-    const uint32_t bytes = r < R ? (uint32_t)C * 2u : 0u;  // nothing is read beyond the last row
-    if (r >= R) r = 0;
-    const __amdgpu_buffer_rsrc_t rsD = make_rsrc(dh + r * lddh, bytes), rsA = make_rsrc(h1 + r * ld1, bytes),
-                                 rsB = make_rsrc(h3 + r * ld3, bytes);
-#pragma unroll
-    for (int j = 0; j < NCHW; ++j) {
-      d[j] = load16_nt(rsD, (uint32_t)col_of(j) * 2u, 0);
-      a[j] = load16_nt(rsA, (uint32_t)col_of(j) * 2u, 0);
-      b[j] = load16_nt(rsB, (uint32_t)col_of(j) * 2u, 0);
-    }
-  };
-  request(blockIdx.x);
   int it = 0;
   for (int64_t r = blockIdx.x; r < R; r += gridDim.x, ++it) {
-    const __amdgpu_buffer_rsrc_t rsG1 = make_rsrc(g1out + r * ldg, (uint32_t)C * 2u), rsG3 = make_rsrc(g3out + r * ldg, (uint32_t)C * 2u);
     v4i g1[NCHW], g3[NCHW];
     uint32_t m1 = 0, m3 = 0;
 #pragma unroll
     for (int j = 0; j < NCHW; ++j) {
       const int c = col_of(j);
+      v4i d = {0, 0, 0, 0}, a = {0, 0, 0, 0}, b = {0, 0, 0, 0};
+      if (c < C) {
+        d = __builtin_nontemporal_load((const v4i *)(dh + r * lddh + c));
+        a = __builtin_nontemporal_load((const v4i *)(h1 + r * ld1 + c));
+        b = __builtin_nontemporal_load((const v4i *)(h3 + r * ld3 + c));
+      }
 #pragma unroll
       for (int k = 0; k < 4; ++k) {
         uint32_t x1, x3;
-        gate_bwd2((uint32_t)d[j][k], (uint32_t)a[j][k], (uint32_t)b[j][k], x1, x3);
+        gate_bwd2((uint32_t)d[k], (uint32_t)a[k], (uint32_t)b[k], x1, x3);
         g1[j][k] = (int)x1;
         g3[j][k] = (int)x3;
         m1 = pk_absmax_u16(m1, x1);
@@ -255,8 +217,10 @@ __global__ __launch_bounds__(BLOCK, BLOCK / 128) void swiglu_bwd_cast_rowwise_ke
         lds_cm1[c / 8] = o1;
         lds_cm3[c / 8] = o3;
       }
-      store16_nt(rsG1, (uint32_t)c * 2u, g1[j]);  // dropped at or beyond column C
-      store16_nt(rsG3, (uint32_t)c * 2u, g3[j]);
+      if (c < C) {
+        __builtin_nontemporal_store(g1[j], (v4i *)(g1out + r * ldg + c));
+        __builtin_nontemporal_store(g3[j], (v4i *)(g3out + r * ldg + c));
+      }
     }
     m1 = wave_max_u32(max(m1 & 0xffffu, m1 >> 16));
     m3 = wave_max_u32(max(m3 & 0xffffu, m3 >> 16));
@@ -265,10 +229,9 @@ __global__ __launch_bounds__(BLOCK, BLOCK / 128) void swiglu_bwd_cast_rowwise_ke
       red[it & 1][1][wave] = m3;
     }
     __syncthreads();
-    request(r + gridDim.x);
     uint32_t bits1 = 0, bits3 = 0;
 #pragma unroll
-    for (int w = 0; w < WAVES; ++w) {
+    for (int w = 0; w < kGateWaves; ++w) {
       bits1 = max(bits1, red[it & 1][0][w]);
       bits3 = max(bits3, red[it & 1][1][w]);
     }
@@ -278,21 +241,14 @@ __global__ __launch_bounds__(BLOCK, BLOCK / 128) void swiglu_bwd_cast_rowwise_ke
       scale3[r] = rs3.s;
     }
     uint8_t *q1row = q1 + r * ldq, *q3row = q3 + r * ldq;
-    const __amdgpu_buffer_rsrc_t rsQ1 = make_rsrc(q1row, (uint32_t)C), rsQ3 = make_rsrc(q3row, (uint32_t)C);
 #pragma unroll
     for (int j = 0; j < NCHW; ++j) {
-      store8_nt(rsQ1, (uint32_t)col_of(j), cvt8(g1[j], rs1.recip));
-      store8_nt(rsQ3, (uint32_t)col_of(j), cvt8(g3[j], rs3.recip));
-    }
-    if (!(rs1.finite && rs3.finite)) {
-      // A row with a non-finite amax: its bytes are redone with the integer conversion, from the gradients this
-      // thread has just stored (same columns), and replace the ones above.  Kept out of the common path as one small
-      // loop: unrolled beside it, the conversion's temporaries pushed loop invariants into scratch memory, whose
-      // reloads wait for every outstanding load.
-#pragma unroll 1
-      for (int c = threadIdx.x * 8; c < C; c += BLOCK * 8) {
-        if (!rs1.finite) *(v2i *)(q1row + c) = cvt8_slow(*(const v4i *)(g1out + r * ldg + c), rs1.recip);
-        if (!rs3.finite) *(v2i *)(q3row + c) = cvt8_slow(*(const v4i *)(g3out + r * ldg + c), rs3.recip);
+      const int c = col_of(j);
+      if (c < C) {
+        if (rs1.finite) __builtin_nontemporal_store(cvt8(g1[j], rs1.recip), (v2i *)(q1row + c));
+        else *(v2i *)(q1row + c) = cvt8_slow(g1[j], rs1.recip);
+        if (rs3.finite) __builtin_nontemporal_store(cvt8(g3[j], rs3.recip), (v2i *)(q3row + c));
+        else *(v2i *)(q3row + c) = cvt8_slow(g3[j], rs3.recip);
       }
     }
   }
@@ -308,7 +264,6 @@ __global__ __launch_bounds__(BLOCK, BLOCK / 128) void swiglu_bwd_cast_rowwise_ke
       }
     }
   }
-#endif
 }
 
 // Wide rows (ffn dimensions beyond what a 256-thread workgroup holds in
@@ -532,41 +487,48 @@ static int launch_bwd_wide(const void *dh, const void *h1, const void *h3, int64
   return L8_OK;
 }
 
-template <int NCHW, int BLOCK>
+template <int NCHW>
 static int launch_fwd(const void *h1, const void *h3, int64_t R, int64_t C, int64_t ld1, int64_t ld3, void *h, int64_t ldh,
                       void *q, int64_t ldq, float *scale, void *amax, float *col_amax, void *ws, hipStream_t st) {
   const int64_t blocks = gate_blocks(R);
   if (col_amax) {
-    const size_t lds = fwd_colmax_in_lds<NCHW, BLOCK>() ? (size_t)C * 2 : 0;
-    hipLaunchKernelGGL((swiglu_cast_rowwise_kernel<NCHW, true, BLOCK>), dim3((unsigned)blocks), dim3(BLOCK), lds, st,
+    const size_t lds = colmax_in_lds<NCHW, 1>() ? (size_t)C * 2 : 0;
+    if (lds > 48 * 1024) {  // above the default limit for dynamic LDS; idempotent
+      static bool raised[kMaxDev] = {};
+      const int slot = device_slot();
+      if (slot < 0 || !raised[slot])
+        L8_HIP(hipFuncSetAttribute((const void *)swiglu_cast_rowwise_kernel<NCHW, true>, hipFuncAttributeMaxDynamicSharedMemorySize, 64 * 1024));
+      if (slot >= 0) raised[slot] = true;
+    }
+    hipLaunchKernelGGL((swiglu_cast_rowwise_kernel<NCHW, true>), dim3((unsigned)blocks), dim3(kGateBlock), lds, st,
                        (const uint16_t *)h1, (const uint16_t *)h3, R, (int)C, ld1, ld3, (uint16_t *)h, ldh, (uint8_t *)q, ldq,
                        scale, (uint16_t *)amax, (uint16_t *)ws, l8::scale_rule());
     L8_HIP(hipGetLastError());
     return fold_colmax(ws, blocks, C, col_amax, st);
   }
-  hipLaunchKernelGGL((swiglu_cast_rowwise_kernel<NCHW, false, BLOCK>), dim3((unsigned)blocks), dim3(BLOCK), 0, st,
+  hipLaunchKernelGGL((swiglu_cast_rowwise_kernel<NCHW, false>), dim3((unsigned)blocks), dim3(kGateBlock), 0, st,
                      (const uint16_t *)h1, (const uint16_t *)h3, R, (int)C, ld1, ld3, (uint16_t *)h, ldh, (uint8_t *)q, ldq,
                      scale, (uint16_t *)amax, (uint16_t *)nullptr, l8::scale_rule());
   L8_HIP(hipGetLastError());
   return L8_OK;
 }
 
-template <int NCHW, int BLOCK>
+template <int NCHW>
 static int launch_bwd(const void *dh, const void *h1, const void *h3, int64_t R, int64_t C, int64_t lddh, int64_t ld1,
                       int64_t ld3, void *g1, void *g3, int64_t ldg, void *q1, void *q3, int64_t ldq, float *s1, float *s3,
                       float *ca1, float *ca3, void *ws, hipStream_t st) {
   const int64_t blocks = gate_blocks(R);
   if (ca1) {
     uint16_t *w1 = (uint16_t *)ws, *w3 = w1 + blocks * C;
-    const size_t lds = bwd_colmax_in_lds<NCHW, BLOCK>() ? (size_t)C * 4 : 0;
+    const size_t lds = colmax_in_lds<NCHW, 2>() ? (size_t)C * 4 : 0;
     if (lds > 48 * 1024) {  // above the default limit for dynamic LDS; idempotent
       static bool raised[kMaxDev] = {};
       const int slot = device_slot();
       if (slot < 0 || !raised[slot])
-        L8_HIP(hipFuncSetAttribute((const void *)swiglu_bwd_cast_rowwise_kernel<NCHW, true, BLOCK>, hipFuncAttributeMaxDynamicSharedMemorySize, 64 * 1024));
+        L8_HIP(hipFuncSetAttribute((const void *)swiglu_bwd_cast_rowwise_kernel<NCHW, true>, hipFuncAttributeMaxDynamicSharedMemorySize, 64 * 1024));
       if (slot >= 0) raised[slot] = true;
     }
-    hipLaunchKernelGGL((swiglu_bwd_cast_rowwise_kernel<NCHW, true, BLOCK>), dim3((unsigned)blocks), dim3(BLOCK), lds, st,
+    hipLaunchKernelGGL((swiglu_bwd_cast_rowwise_kernel<NCHW, true>), dim3((unsigned)blocks), dim3(kGateBlock), lds, st,
                        (const uint16_t *)dh, (const uint16_t *)h1, (const uint16_t *)h3, R, (int)C, lddh, ld1, ld3,
                        (uint16_t *)g1, (uint16_t *)g3, ldg, (uint8_t *)q1, (uint8_t *)q3, ldq, s1, s3, w1, w3, l8::scale_rule());
     L8_HIP(hipGetLastError());
@@ -574,7 +536,7 @@ static int launch_bwd(const void *dh, const void *h1, const void *h3, int64_t R,
     if (rc != L8_OK) return rc;
     return fold_colmax(w3, blocks, C, ca3, st);
   }
-  hipLaunchKernelGGL((swiglu_bwd_cast_rowwise_kernel<NCHW, false, BLOCK>), dim3((unsigned)blocks), dim3(BLOCK), 0, st,
+  hipLaunchKernelGGL((swiglu_bwd_cast_rowwise_kernel<NCHW, false>), dim3((unsigned)blocks), dim3(kGateBlock), 0, st,
                      (const uint16_t *)dh, (const uint16_t *)h1, (const uint16_t *)h3, R, (int)C, lddh, ld1, ld3,
                      (uint16_t *)g1, (uint16_t *)g3, ldg, (uint8_t *)q1, (uint8_t *)q3, ldq, s1, s3, (uint16_t *)nullptr,
                      (uint16_t *)nullptr, l8::scale_rule());
@@ -613,13 +575,13 @@ extern "C" int l8_swiglu_cast_rowwise(const void *h1, const void *h3, int64_t R,
                "l8_swiglu_cast_rowwise: col_amax needs a 16-byte aligned workspace of %lld bytes", (long long)need);
   }
   hipStream_t st = (hipStream_t)stream;
-  const int64_t nch = (C + 511) / 512;  // 512-column chunks of a row, one per wave and pass
-#define L8_FWD(N, B) return launch_fwd<N, B>(h1, h3, R, C, ld1, ld3, h, ldh, q, ldq, scale, amax, col_amax, workspace, st)
-  if (nch <= 4) L8_FWD(1, 256);
-  if (nch <= 8) L8_FWD(2, 256);
-  if (nch <= 16) L8_FWD(2, 512);
-  if (nch <= 24) L8_FWD(3, 512);
-  if (nch <= 32) L8_FWD(4, 512);
+  const int64_t nchw = ((C + 511) / 512 + kGateWaves - 1) / kGateWaves;
+#define L8_FWD(N) return launch_fwd<N>(h1, h3, R, C, ld1, ld3, h, ldh, q, ldq, scale, amax, col_amax, workspace, st)
+  if (nchw <= 1) L8_FWD(1);
+  if (nchw <= 2) L8_FWD(2);
+  if (nchw <= 4) L8_FWD(4);
+  if (nchw <= 6) L8_FWD(6);
+  if (nchw <= 8) L8_FWD(8);
 #undef L8_FWD
   return launch_fwd_wide(h1, h3, R, C, ld1, ld3, h, ldh, q, ldq, scale, amax, col_amax, workspace, st);
 }
@@ -645,14 +607,14 @@ extern "C" int l8_swiglu_bwd_cast_rowwise(const void *dh, const void *h1, const 
                "l8_swiglu_bwd_cast_rowwise: column amaxes need a 16-byte aligned workspace of %lld bytes", (long long)need);
   }
   hipStream_t st = (hipStream_t)stream;
-  const int64_t nch = (C + 511) / 512;  // 512-column chunks of a row, one per wave and pass
-#define L8_BWD(N, B)                                                                                                  \
-  return launch_bwd<N, B>(dh, h1, h3, R, C, lddh, ld1, ld3, g1, g3, ldg, q1, q3, ldq, scale1, scale3, col_amax1, col_amax3, \
-                          workspace, st)
-  if (nch <= 4) L8_BWD(1, 256);
-  if (nch <= 8) L8_BWD(2, 256);
-  if (nch <= 16) L8_BWD(2, 512);
-  if (nch <= 24) L8_BWD(3, 512);
+  const int64_t nchw = ((C + 511) / 512 + kGateWaves - 1) / kGateWaves;
+#define L8_BWD(N)                                                                                                  \
+  return launch_bwd<N>(dh, h1, h3, R, C, lddh, ld1, ld3, g1, g3, ldg, q1, q3, ldq, scale1, scale3, col_amax1, col_amax3, \
+                       workspace, st)
+  if (nchw <= 1) L8_BWD(1);
+  if (nchw <= 2) L8_BWD(2);
+  if (nchw <= 4) L8_BWD(4);
+  if (nchw <= 6) L8_BWD(6);
 #undef L8_BWD
   return launch_bwd_wide(dh, h1, h3, R, C, lddh, ld1, ld3, g1, g3, ldg, q1, q3, ldq, scale1, scale3, col_amax1, col_amax3,
                          workspace, st);
