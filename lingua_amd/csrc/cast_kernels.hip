@@ -442,25 +442,30 @@ __global__ __launch_bounds__(256) void cast_rowwise_given_amax_kernel(const uint
 // dword and writes it to the transposed tile in LDS; the tile is then read
 // back as 16-byte row segments and stored as 256-byte runs of the output rows.
 // ---------------------------------------------------------------------------
-#ifndef L8_TC
-#define L8_TC 64
-#endif
-#ifndef L8_TU
-#define L8_TU 2
-#endif
-constexpr int kTC = L8_TC;                   // columns of x per tile
-constexpr int kCCH = kTC / 8;                // 8-column chunks per tile row
-constexpr int kRG = 256 / kCCH;              // 4-row groups covered by the 256 threads in one pass
-constexpr int kTU = L8_TU;                   // passes (4-row units per thread)
-constexpr int kTR = kRG * 4 * kTU;           // rows of x per tile
-[[maybe_unused]] constexpr int kTStride = kTR + 16;           // LDS row stride in bytes
+// Tile shapes: TC columns x (256 / (TC / 8)) * 4 * TU rows.  128 x 128 (TC 128, TU 2) is the one used; 64 x 128 (TC 64,
+// TU 1) for tensors with too few 128 x 128 tiles to fill the chip.  Inside the MLP step, against the 64 x 256 tile this
+// kernel had before: [16384,4096] 39.1 -> 37.3 us, [16384,11008] 110.1 -> 107.9, weights 28.0 -> 28.0; Llama-1B shapes:
+// [16384,8192] 80.1 -> 73.8, [16384,2048] 21.0 -> 21.1, [8192,2048] 12.4 -> 11.8, [2048,2048] 5.2 -> 4.9 (64 x 128).
+// 128 x 256 was another 1-5 % ahead on the two widest activations and 4 % behind on every weight.
+template <int TC, int TU>
+struct TransposeTile {
+  static constexpr int kTC = TC;                  // columns of x per tile
+  static constexpr int kCCH = TC / 8;             // 8-column chunks per tile row
+  static constexpr int kRG = 256 / kCCH;          // 4-row groups covered by the 256 threads in one pass
+  static constexpr int kTU = TU;                  // passes (4-row units per thread)
+  static constexpr int kTR = kRG * 4 * TU;        // rows of x per tile
+  static constexpr int kTStride = kTR + 16;       // LDS row stride in bytes
+};
+constexpr int kMaxTileRows = 256;                 // no tile is taller (bounds the row stride the host accepts)
 
-template <bool PER_COL>
+template <bool PER_COL, int TC, int TU>
 __global__ __launch_bounds__(256) void cast_transposed_kernel(
     const uint16_t *__restrict__ x, int64_t R, int C, int64_t ldx, const void *__restrict__ amax_scalar, int amax_f32,
     const uint32_t *__restrict__ col_amax, uint8_t *__restrict__ q, int64_t ldq, float *__restrict__ scale,
     int vec_store, int scale_rule) {
 #if defined(__HIP_DEVICE_COMPILE__)  // the buffer-resource type exists in the device pass only
+  using T = TransposeTile<TC, TU>;
+  constexpr int kTC = T::kTC, kCCH = T::kCCH, kRG = T::kRG, kTU = T::kTU, kTR = T::kTR, kTStride = T::kTStride;
   __shared__ __attribute__((aligned(16))) uint8_t tile[kTC * kTStride];
   __shared__ float recips[kTC];
   const int t = threadIdx.x;
@@ -833,23 +838,34 @@ extern "C" int l8_amax_reduce(const void *amax, int64_t n, void *amax_out, void 
   return L8_OK;
 }
 
-static int launch_transposed(bool per_col, const void *x, int64_t R, int64_t C, int64_t ldx, const void *amax,
-                             int amax_f32, const float *col_amax, void *q, int64_t ldq, float *scale, hipStream_t st) {
-  const int64_t gx = ((C + kTC - 1) / kTC) * ((R + kTR - 1) / kTR), gy = 1;
+template <int TC, int TU>
+static int launch_transposed_tile(bool per_col, const void *x, int64_t R, int64_t C, int64_t ldx, const void *amax,
+                                  int amax_f32, const float *col_amax, void *q, int64_t ldq, float *scale, hipStream_t st) {
+  using T = TransposeTile<TC, TU>;
+  static_assert(T::kTR <= kMaxTileRows, "the row-stride limit assumes no taller tile");
+  const int64_t gx = ((C + T::kTC - 1) / T::kTC) * ((R + T::kTR - 1) / T::kTR);
   L8_REQUIRE(gx < (1LL << 31), "transposed cast: shape too large (%lld x %lld)", (long long)R, (long long)C);
-  // a tile's 256 rows within 1 GiB: then no sum of a lane's offset (up to twice the tile) and a row's scalar offset wraps
-  L8_REQUIRE((int64_t)kTR * ldx * 2 < (1LL << 30), "transposed cast: row stride too large (%lld elements)", (long long)ldx);
   const int vec = (ldq % 16 == 0 && aligned(q, 16)) ? 1 : 0;
   if (per_col)
-    hipLaunchKernelGGL((cast_transposed_kernel<true>), dim3((unsigned)gx, (unsigned)gy), dim3(256), 0, st,
+    hipLaunchKernelGGL((cast_transposed_kernel<true, TC, TU>), dim3((unsigned)gx), dim3(256), 0, st,
                        (const uint16_t *)x, R, (int)C, ldx, (const void *)nullptr, 0, (const uint32_t *)col_amax,
                        (uint8_t *)q, ldq, scale, vec, l8::scale_rule());
   else
-    hipLaunchKernelGGL((cast_transposed_kernel<false>), dim3((unsigned)gx, (unsigned)gy), dim3(256), 0, st,
+    hipLaunchKernelGGL((cast_transposed_kernel<false, TC, TU>), dim3((unsigned)gx), dim3(256), 0, st,
                        (const uint16_t *)x, R, (int)C, ldx, amax, amax_f32, (const uint32_t *)nullptr,
                        (uint8_t *)q, ldq, scale, vec, l8::scale_rule());
   L8_HIP(hipGetLastError());
   return L8_OK;
+}
+
+static int launch_transposed(bool per_col, const void *x, int64_t R, int64_t C, int64_t ldx, const void *amax,
+                             int amax_f32, const float *col_amax, void *q, int64_t ldq, float *scale, hipStream_t st) {
+  // a tile's rows within 1 GiB: then no sum of a lane's offset (up to twice the tile) and a row's scalar offset wraps
+  L8_REQUIRE((int64_t)kMaxTileRows * ldx * 2 < (1LL << 30), "transposed cast: row stride too large (%lld elements)", (long long)ldx);
+  const int64_t tiles128 = ((C + 127) / 128) * ((R + 127) / 128);
+  if (tiles128 < 4 * (int64_t)num_cus())  // too few 128 x 128 tiles for four workgroups per compute unit
+    return launch_transposed_tile<64, 1>(per_col, x, R, C, ldx, amax, amax_f32, col_amax, q, ldq, scale, st);
+  return launch_transposed_tile<128, 2>(per_col, x, R, C, ldx, amax, amax_f32, col_amax, q, ldq, scale, st);
 }
 
 extern "C" int l8_cast_tensorwise(const void *x, int64_t R, int64_t C, int64_t ldx, const void *amax, int amax_dtype,

@@ -203,6 +203,45 @@ def test_transposed_casts_with_a_nonfinite_amax_over_several_tiles(bad, amax_dty
         assert bits_equal(s[fin], so[fin])
 
 
+@pytest.mark.parametrize("ldq_pad", [0, 7])
+def test_transposed_casts_with_ragged_edges_on_the_large_tile(ldq_pad):
+    """Tensors with at least four 128 x 128 tiles per compute unit take the 128 x 128 tile (smaller ones a 64 x 128
+    tile, which the random-shape sweep covers): rows and columns that are not multiples of the tile, a padded input
+    row stride, an output row stride that rules out 16-byte stores, and one column with a non-finite amax."""
+    from lingua_amd import _lib
+    lib = _lib.load()
+    R, C, ldx = 4100, 4104, 4112
+    g = torch.Generator().manual_seed(21)
+    xb = torch.randn(R, ldx, generator=g).to(torch.bfloat16)
+    xb[:, C:] = 3.0e38                      # padding columns must not be read
+    xb[17, 130] = float("inf")
+    x = xb.cuda()
+    xc = xb[:, :C].contiguous()
+    ldq = (R + 15) // 16 * 16 + ldq_pad
+    st = torch.cuda.current_stream().cuda_stream
+    col = torch.zeros(C, dtype=torch.float32, device="cuda")
+    _lib.check(lib.l8_col_amax(x.data_ptr(), R, C, ldx, col.data_ptr(), st), "l8_col_amax")
+    q = torch.full((C, ldq), 0x55, dtype=torch.uint8, device="cuda")
+    s = torch.empty(C, dtype=torch.float32, device="cuda")
+    _lib.check(lib.l8_cast_colwise_transposed(x.data_ptr(), R, C, ldx, col.data_ptr(), q.data_ptr(), ldq, s.data_ptr(), st),
+               "l8_cast_colwise_transposed")
+    wq, ws = oracle.cast_colwise_transposed(xc)
+    assert fp8_equal_mod_nan_sign(q.cpu()[:, :R], wq)
+    assert (q.cpu()[:, R:] == 0x55).all()
+    fin = ws.isfinite()
+    assert int((~fin).sum()) == 1 and not fin[130] and bits_equal(s.cpu()[fin], ws[fin])
+    amax = oracle.amax_of_amaxes(oracle.row_amax(xc[:, :128]))      # a finite amax that does not bound the tensor
+    q = torch.full((C, ldq), 0x55, dtype=torch.uint8, device="cuda")
+    s1 = torch.empty(1, dtype=torch.float32, device="cuda")
+    xfin = xb.clone()
+    xfin[17, 130] = 1.0
+    xfin[:, :C] = xfin[:, :C].clamp(-float(amax.float()), float(amax.float()))
+    _lib.check(lib.l8_cast_tensorwise(xfin.cuda().data_ptr(), R, C, ldx, amax.cuda().data_ptr(), 0, 1, q.data_ptr(), ldq,
+                                      s1.data_ptr(), st), "l8_cast_tensorwise")
+    wq, ws = oracle.cast_tensorwise(xfin[:, :C].contiguous(), amax, transpose=True)
+    assert torch.equal(q.cpu()[:, :R], wq) and (q.cpu()[:, R:] == 0x55).all() and bits_equal(s1.cpu(), ws.reshape(-1))
+
+
 from bench_workloads import outlier_stress_input  # noqa: E402
 
 
