@@ -91,7 +91,7 @@ __global__ __launch_bounds__(kRowBlock, 2) void cast_rowwise_kernel(
     uint8_t *qrow = q ? q + r * ldq : nullptr;
     const __amdgpu_buffer_rsrc_t rsQ = make_rsrc(qrow, q ? (uint32_t)C : 0u);  // stores beyond column C, or without q, are dropped
 #pragma unroll
-    for (int j = 0; j < NCH; ++j) store8_nt(rsQ, (uint32_t)(j * 512 + lane * 8), cvt8(cur[j], recip));
+    for (int j = 0; j < NCH; ++j) store8(rsQ, (uint32_t)(j * 512 + lane * 8), cvt8(cur[j], recip));
     if (q && !finite) {
       // a row with a non-finite amax: redone from memory with the integer conversion, replacing the bytes above (one
       // small loop beside the common path instead of NCH unrolled copies of that conversion inside it)
@@ -197,7 +197,7 @@ __global__ __launch_bounds__(kRowBlock, (NCHW <= 4 ? 4 : (NCHW <= 8 ? 2 : 1))) v
     uint8_t *qrow = q ? q + r * ldq : nullptr;
     const __amdgpu_buffer_rsrc_t rsQ = make_rsrc(qrow, q ? (uint32_t)C : 0u);  // stores beyond column C, or without q, are dropped
 #pragma unroll
-    for (int j = 0; j < NCHW; ++j) store8_nt(rsQ, (uint32_t)col_of(j), cvt8(cur[j], recip));
+    for (int j = 0; j < NCHW; ++j) store8(rsQ, (uint32_t)col_of(j), cvt8(cur[j], recip));
     if (q && !finite) {  // non-finite amax: redone from memory with the integer conversion, as in cast_rowwise_kernel
 #pragma unroll 1
       for (int c = threadIdx.x * 8; c < C; c += kRowBlock * 8)
@@ -447,6 +447,10 @@ __global__ __launch_bounds__(256) void cast_rowwise_given_amax_kernel(const uint
 // kernel had before: [16384,4096] 39.1 -> 37.3 us, [16384,11008] 110.1 -> 107.9, weights 28.0 -> 28.0; Llama-1B shapes:
 // [16384,8192] 80.1 -> 73.8, [16384,2048] 21.0 -> 21.1, [8192,2048] 12.4 -> 11.8, [2048,2048] 5.2 -> 4.9 (64 x 128).
 // 128 x 256 was another 1-5 % ahead on the two widest activations and 4 % behind on every weight.
+// The loads are non-temporal, the stores are not: a workgroup writes 128-byte pieces of 128 output rows, the pieces
+// next to them come from other workgroups a little later, and ordinary stores leave it to the L2 to write neighbours
+// back together.  Inside the MLP step, ordinary against non-temporal stores: [16384,11008] 99.4 against 108.4 us,
+// [16384,4096] 35.5 against 37.2, weights 26.2 against 27.7; ordinary loads instead cost 2-4 %.
 template <int TC, int TU>
 struct TransposeTile {
   static constexpr int kTC = TC;                  // columns of x per tile
@@ -601,7 +605,7 @@ __global__ __launch_bounds__(256) void cast_transposed_kernel(
       const v4i v = *(const v4i *)(tile + oc * kTStride + seg * 16);
       uint8_t *dst = q + (int64_t)col * ldq + r;
       if (vec_store && r + 16 <= R) {
-        __builtin_nontemporal_store(v, (v4i *)dst);
+        *(v4i *)dst = v;  // not a streaming store: see the note on the tile shapes
       } else {
         const uint8_t *src = tile + oc * kTStride + seg * 16;
         for (int b = 0; b < 16 && r + b < R; ++b) dst[b] = src[b];

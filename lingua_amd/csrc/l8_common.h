@@ -181,9 +181,10 @@ L8_DEV __amdgpu_buffer_rsrc_t make_rsrc(const void *p, uint32_t bytes) {
 L8_DEV v4i load16_nt(__amdgpu_buffer_rsrc_t rs, uint32_t voff, uint32_t soff) {
   return __builtin_amdgcn_raw_buffer_load_b128(rs, (int)voff, (int)soff, 2 /* cache policy: non-temporal */);
 }
-// one 8-byte non-temporal store at lane offset voff (dropped beyond the descriptor's range)
-L8_DEV void store8_nt(__amdgpu_buffer_rsrc_t rs, uint32_t voff, v2i data) {
-  __builtin_amdgcn_raw_buffer_store_b64(data, rs, (int)voff, 0, 2);
+// One 8-byte store at lane offset voff (dropped beyond the descriptor's range).  An ordinary store, not a non-temporal
+// one: inside the MLP step the row-wise casts ran 2-5 % faster with it (the output is the next GEMM's operand).
+L8_DEV void store8(__amdgpu_buffer_rsrc_t rs, uint32_t voff, v2i data) {
+  __builtin_amdgcn_raw_buffer_store_b64(data, rs, (int)voff, 0, 0);
 }
 #endif
 
