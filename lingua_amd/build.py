@@ -74,6 +74,14 @@ def _check_usage(usage) -> None:
     bad = [f"{name}: {u}" for name, u in stream.items() if (u["ScratchSize"] or u["VGPRs Spill"])]
     if bad:
         raise RuntimeError("the persistent GEMM kernel must not use scratch memory:\n  " + "\n  ".join(bad))
+    # The cast, gate and norm kernels stream memory with several loads in flight per lane; a reload from scratch memory
+    # waits for every one of them (loads retire in order).  None of them needs scratch, so one that starts to is a
+    # regression of the source.  (The plain GEMM kernels of the non-default tile configurations spill a few registers
+    # by design and are not checked.)
+    bad = [f"{name}: {u}" for name, u in usage.items()
+           if "gemm_nt" not in name and (u.get("ScratchSize") or u.get("VGPRs Spill"))]
+    if bad:
+        raise RuntimeError("memory-streaming kernels must not use scratch memory:\n  " + "\n  ".join(bad))
 
 
 def build(verbose: bool = False) -> str:

@@ -229,6 +229,11 @@ def test_build_refuses_a_persistent_gemm_kernel_that_uses_scratch():
         bad["_ZN2l821gemm_nt_stream_kernelILi4ELb0ELb0EEEvNS_8GemmArgsE"][field] = 12
         with pytest.raises(RuntimeError):
             build._check_usage(bad)
+    # the memory-streaming kernels (casts, gate, norm) must not use scratch memory either
+    spilled = {k: dict(v) for k, v in ok.items()}
+    spilled["_ZN2l822cast_rowwise_wg_kernelILi6ELb1EEEvPKtlilPhlPfPtS5_i"] = {"VGPRs": 128, "ScratchSize": 8, "VGPRs Spill": 1}
+    with pytest.raises(RuntimeError, match="streaming"):
+        build._check_usage(spilled)
     # a check that finds nothing to check must fail too: no remark parsed at all, or one without the figures
     with pytest.raises(RuntimeError):
         build._check_usage({})
