@@ -447,6 +447,10 @@ __global__ __launch_bounds__(256) void cast_rowwise_given_amax_kernel(const uint
 // kernel had before: [16384,4096] 39.1 -> 37.3 us, [16384,11008] 110.1 -> 107.9, weights 28.0 -> 28.0; Llama-1B shapes:
 // [16384,8192] 80.1 -> 73.8, [16384,2048] 21.0 -> 21.1, [8192,2048] 12.4 -> 11.8, [2048,2048] 5.2 -> 4.9 (64 x 128).
 // 128 x 256 was another 1-5 % ahead on the two widest activations and 4 % behind on every weight.
+// Tensors of at least 16384 rows and 8192 columns take 128 x 256 (TU 4): over 26 activation shapes, each timed right
+// behind the kernel that produces it, 128 x 128 and 128 x 256 are within 1-3 % of each other there except at 11008
+// columns (the 7B ffn width), where 128 x 128 alone falls off -- [16384,11008] 100 against 90 us, [32768,11008] 206
+// against 187 -- while 10880, 11136, 11264 and 11520 columns show nothing of the kind.
 // The loads are non-temporal, the stores are not: a workgroup writes 128-byte pieces of 128 output rows, the pieces
 // next to them come from other workgroups a little later, and ordinary stores leave it to the L2 to write neighbours
 // back together.  Inside the MLP step, ordinary against non-temporal stores: [16384,11008] 99.4 against 108.4 us,
@@ -869,6 +873,8 @@ static int launch_transposed(bool per_col, const void *x, int64_t R, int64_t C, 
   const int64_t tiles128 = ((C + 127) / 128) * ((R + 127) / 128);
   if (tiles128 < 4 * (int64_t)num_cus())  // too few 128 x 128 tiles for four workgroups per compute unit
     return launch_transposed_tile<64, 1>(per_col, x, R, C, ldx, amax, amax_f32, col_amax, q, ldq, scale, st);
+  if (R >= 16384 && C >= 8192)  // the large activations: see the note on the tile shapes
+    return launch_transposed_tile<128, 4>(per_col, x, R, C, ldx, amax, amax_f32, col_amax, q, ldq, scale, st);
   return launch_transposed_tile<128, 2>(per_col, x, R, C, ldx, amax, amax_f32, col_amax, q, ldq, scale, st);
 }
 

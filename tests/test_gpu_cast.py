@@ -242,6 +242,33 @@ def test_transposed_casts_with_ragged_edges_on_the_large_tile(ldq_pad):
     assert torch.equal(q.cpu()[:, :R], wq) and (q.cpu()[:, R:] == 0x55).all() and bits_equal(s1.cpu(), ws.reshape(-1))
 
 
+def test_transposed_casts_with_ragged_edges_on_the_tall_tile():
+    """Tensors of at least 16384 rows and 8192 columns take a 128 x 256 tile: same edge cases as for the other tiles,
+    the whole output against the C oracle."""
+    from lingua_amd import _lib
+    lib = _lib.load()
+    R, C, ldx = 16390, 8200, 8208
+    g = torch.Generator().manual_seed(22)
+    xb = torch.randn(R, ldx, generator=g).to(torch.bfloat16)
+    xb[:, C:] = 3.0e38                      # padding columns must not be read
+    xb[16389, 8199] = float("nan")
+    x = xb.cuda()
+    xc = xb[:, :C].contiguous()
+    st = torch.cuda.current_stream().cuda_stream
+    col = torch.zeros(C, dtype=torch.float32, device="cuda")
+    _lib.check(lib.l8_col_amax(x.data_ptr(), R, C, ldx, col.data_ptr(), st), "l8_col_amax")
+    for ldq in (16400, 16391):              # 16-byte stores, byte stores
+        q = torch.full((C, ldq), 0x55, dtype=torch.uint8, device="cuda")
+        s = torch.empty(C, dtype=torch.float32, device="cuda")
+        _lib.check(lib.l8_cast_colwise_transposed(x.data_ptr(), R, C, ldx, col.data_ptr(), q.data_ptr(), ldq, s.data_ptr(), st),
+                   "l8_cast_colwise_transposed")
+        wq, ws = oracle.cast_colwise_transposed(xc)
+        assert fp8_equal_mod_nan_sign(q[:, :R].cpu(), wq), ldq
+        assert bool((q[:, R:] == 0x55).all()), ldq
+        fin = ws.isfinite()
+        assert int((~fin).sum()) == 1 and not fin[8199] and bits_equal(s.cpu()[fin], ws[fin]), ldq
+
+
 from bench_workloads import outlier_stress_input  # noqa: E402
 
 
